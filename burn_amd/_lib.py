@@ -14,9 +14,9 @@ LIB_PATH = os.path.join(HERE, "libburnq_mi355.so")
 MAX_RANK = 8
 
 # bq_status
-OK, ERR_NULL, ERR_UNSUPPORTED_SCHEME, ERR_SHAPE, ERR_DTYPE, ERR_HIP, ERR_SIZE, ERR_UNSUPPORTED_OP = range(8)
+OK, ERR_NULL, ERR_UNSUPPORTED_SCHEME, ERR_SHAPE, ERR_DTYPE, ERR_HIP, ERR_SIZE, ERR_UNSUPPORTED_OP, ERR_NONFINITE = range(9)
 STATUS_NAMES = ["OK", "ERR_NULL", "ERR_UNSUPPORTED_SCHEME", "ERR_SHAPE", "ERR_DTYPE", "ERR_HIP",
-                "ERR_SIZE", "ERR_UNSUPPORTED_OP"]
+                "ERR_SIZE", "ERR_UNSUPPORTED_OP", "ERR_NONFINITE"]
 # dtypes
 F32, BF16, QFLOAT = 0, 1, 2
 # scheme enums
@@ -55,6 +55,7 @@ SIGNATURES = {
     "bq_device_sync": (_i32, [_vp]),
     "bq_device_stream": (_vp, [_vp]),
     "bq_device_trim": (_i32, [_vp]),
+    "bq_device_set_validate": (_i32, [_vp, _i32]),
     "bq_timer_start": (_i32, [_vp]),
     "bq_timer_stop": (_i32, [_vp, C.POINTER(C.c_float)]),
     "bq_graph_begin_capture": (_i32, [_vp]),
@@ -92,6 +93,7 @@ SIGNATURES = {
     "bq_q_flip": (_i32, [_vp, C.POINTER(_i32), _i32, _pvp]),
     "bqk_selftest_division": (_i32, [_vp, _vp]),
     "bqk_copy": (_i32, [_vp, _vp, _sz, _vp]),
+    "bqk_lds_request_status": (_i32, [_sz, _sz]),
     "bqk_absmax_f32": (_i32, [_vp, _sz, _vp, _vp]),
     "bqk_quantize_per_tensor_from_absmax": (_i32, [_vp, _sz, _vp, _vp, _i32, _i32, _vp, _vp]),
     "bqk_scales_from_absmax": (_i32, [_vp, _sz, _i32, _vp, _vp]),

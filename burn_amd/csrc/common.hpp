@@ -13,6 +13,7 @@
 #include <string>
 #include <vector>
 
+#include "block_cache.hpp"
 #include "burnq.h"
 
 namespace bq {
@@ -61,12 +62,16 @@ struct bq_device {
   hipStream_t stream = nullptr;
   hipEvent_t ev_start = nullptr, ev_stop = nullptr;
   std::mutex mu;                                  // guards the allocation cache and workspace
-  std::multimap<size_t, void*> free_blocks;       // size -> cached allocation
-  void* workspace = nullptr;                      // split-K partials, absmax cell, counters
+  bq::BlockCache cache;                           // cached allocations, graph-capture bookkeeping
+  void* workspace = nullptr;                      // split-K partials, bf16 copy of an f32 lhs
   size_t workspace_bytes = 0;
   int num_cus = 256;
+  size_t lds_limit = 64 * 1024;                   // largest dynamic LDS request a launch may make
+  std::atomic<bool> validate{false};              // bq_device_set_validate
+  uint32_t* validate_cells = nullptr;             // 4 device counters of the validate mode
 
-  bq_status alloc(size_t bytes, void** out);      // stream-ordered reuse is safe: one stream
+  // *actual receives the size of the block handed out (at least `bytes`); pass it to release().
+  bq_status alloc(size_t bytes, void** out, size_t* actual);  // stream-ordered reuse is safe: one stream
   void release(void* ptr, size_t bytes);
   bq_status ensure_workspace(size_t bytes);
   bq_status trim();
@@ -148,5 +153,15 @@ bool fused_matmul_ok(size_t m, size_t k, size_t n, int lhs_dtype, int value, siz
 
 // dst[0..n) = value, as a kernel (safe to record into a HIP graph, unlike a memset node).
 bq_status launch_fill_u32(uint32_t* dst, size_t n, uint32_t value, hipStream_t stream);
+
+// Host-side guard of a kernel's dynamic LDS request (runtime.cpp). A request beyond what the
+// current device grants is refused here with BQ_ERR_HIP: it must never reach a launch. The first
+// call for a (device, kernel) pair raises the kernel's dynamic-LDS attribute; later ones only check.
+bq_status lds_request_status(size_t bytes, size_t device_limit, const char* what);
+bq_status configure_dynamic_lds(const void* kernel, size_t bytes, const char* what);
+
+// Counts, over n floats, NaNs into counts[0] and infinities into counts[1] (device u32 cells that
+// the kernel adds to; quantize.hip). Used by the validate mode.
+bq_status launch_count_nonfinite(const float* x, size_t n, uint32_t* counts, hipStream_t stream);
 
 }  // namespace bq

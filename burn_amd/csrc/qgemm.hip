@@ -509,12 +509,8 @@ bq_status launch_one(const uint16_t* a, const uint32_t* w, const float* scales, 
   constexpr size_t lds_bytes = 2 * (static_cast<size_t>(BM) + BN) * kRowBytes;
   const bool k_tail = k % (2 * BK) != 0;  // also pads an odd stage count (slices hold even counts)
   auto kernel = k_tail ? qgemm_kernel<VPL, BM, OUT_BF16, true> : qgemm_kernel<VPL, BM, OUT_BF16, false>;
-  static bool configured[2] = {false, false};  // one attribute call per instantiation
-  if (!configured[k_tail]) {
-    BQ_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
-                               hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds_bytes)));
-    configured[k_tail] = true;
-  }
+  // (checked on the host against what the device grants per workgroup; refused, never launched, beyond it)
+  BQ_TRY(configure_dynamic_lds(reinterpret_cast<const void*>(kernel), lds_bytes, "qgemm_kernel"));
   dim3 grid(static_cast<unsigned>((n + BN - 1) / BN), static_cast<unsigned>((m + BM - 1) / BM), slices), tb(gemm_waves(BM, VPL) * kWave);
   hipLaunchKernelGGL(kernel, grid, tb, lds_bytes, st, a, w, scales, m, k, n, nw, bwl2, spr, per_tensor, stages_per_slice, bias, out);
   BQ_HIP(hipGetLastError());

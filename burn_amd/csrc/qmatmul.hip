@@ -559,7 +559,10 @@ __global__ void empty_k_kernel(const float* __restrict__ bias, size_t mn, size_t
 static bq_status q_matmul_core(const void* lhs, int32_t lhs_dtype, size_t m, size_t k, size_t n,
                                const void* w_values, const float* w_scales, int32_t block,
                                int32_t value, int32_t store, const float* bias, int32_t out_dtype, void* out,
-                               void* workspace, size_t workspace_bytes, void* stream) {
+                               void* workspace, size_t workspace_bytes, void* stream, size_t* need_out = nullptr) {
+  // need_out: dry run. The arguments are validated and the kernel is chosen as usual, but nothing is
+  // launched: *need_out receives the scratch bytes that kernel would use.
+  if (need_out) *need_out = 0;
   BQ_NOTNULL(lhs);
   BQ_NOTNULL(w_values);
   BQ_NOTNULL(w_scales);
@@ -586,6 +589,7 @@ static bq_status q_matmul_core(const void* lhs, int32_t lhs_dtype, size_t m, siz
   const uint32_t* w = static_cast<const uint32_t*>(w_values);
 
   if (k == 0) {  // an empty sum, written by a kernel (a memset node must not enter a captured graph)
+    if (need_out) return BQ_OK;
     hipLaunchKernelGGL(empty_k_kernel, dim3(static_cast<unsigned>((m * n + 255) / 256)), dim3(256), 0, st, bias,
                        m * n, n, out_dtype, out);
     BQ_HIP(hipGetLastError());
@@ -602,6 +606,7 @@ static bq_status q_matmul_core(const void* lhs, int32_t lhs_dtype, size_t m, siz
       (reinterpret_cast<uintptr_t>(w_values) & 15u) == 0 &&
       (per_tensor || (reinterpret_cast<uintptr_t>(w_scales) & 15u) == 0)) {
     const size_t need = split_workspace(m, k, n);
+    if (need_out) return *need_out = need, BQ_OK;
     if (workspace == nullptr || workspace_bytes < need)
       BQ_FAIL(BQ_ERR_SIZE, "q_matmul workspace: need %zu bytes, got %zu", need, workspace_bytes);
     float* part = static_cast<float*>(workspace);
@@ -615,6 +620,7 @@ static bq_status q_matmul_core(const void* lhs, int32_t lhs_dtype, size_t m, siz
     const size_t cpl = static_cast<size_t>(gemv1_words(static_cast<int>(vpl))) * vpl;
     GemvPlan p = gemv1_plan(m, k, n, value);
     const size_t need = static_cast<size_t>(p.slices) * m * n * sizeof(float);
+    if (need_out) return *need_out = need, BQ_OK;
     if (workspace == nullptr || workspace_bytes < need)
       BQ_FAIL(BQ_ERR_SIZE, "q_matmul workspace: need %zu bytes, got %zu", need, workspace_bytes);
     float* part = static_cast<float*>(workspace);
@@ -675,6 +681,7 @@ static bq_status q_matmul_core(const void* lhs, int32_t lhs_dtype, size_t m, siz
       !f32_small || (m >= 7 && (per_tensor || bwl2 >= 2) && (reinterpret_cast<uintptr_t>(w_values) & 15u) == 0);
   if (skinny_ok(m, k, n, lhs_dtype, value) && skinny_layout_ok) {
     const size_t need = skinny_workspace(m, k, n, lhs_dtype, value);
+    if (need_out) return *need_out = need, BQ_OK;
     if (workspace == nullptr || workspace_bytes < need)
       BQ_FAIL(BQ_ERR_SIZE, "q_matmul workspace: need %zu bytes, got %zu", need, workspace_bytes);
     float* part = static_cast<float*>(workspace);
@@ -686,6 +693,7 @@ static bq_status q_matmul_core(const void* lhs, int32_t lhs_dtype, size_t m, siz
   if (use_gemv(m, lhs_dtype)) {
     GemvPlan p = gemv_plan(k, n, value);
     const size_t need = static_cast<size_t>(p.slices) * m * n * sizeof(float);
+    if (need_out) return *need_out = need, BQ_OK;
     if (workspace == nullptr || workspace_bytes < need)
       BQ_FAIL(BQ_ERR_SIZE, "q_matmul workspace: need %zu bytes, got %zu", need, workspace_bytes);
     float* part = static_cast<float*>(workspace);
@@ -726,6 +734,7 @@ static bq_status q_matmul_core(const void* lhs, int32_t lhs_dtype, size_t m, siz
 
   if (!qgemm_ok(lhs_dtype, k, n, value, spr))
     BQ_FAIL(BQ_ERR_SHAPE, "the tiled q_matmul needs K %% 8 == 0 and operands under 4 GiB (K = %zu)", k);
+  if (need_out) return *need_out = qgemm_workspace(lhs_dtype, m, k, n), BQ_OK;
   unsigned slices = 1;
   float* part = nullptr;
   BQ_TRY(launch_qgemm(lhs, lhs_dtype, w, w_scales, m, k, n, value, bwl2, spr, per_tensor, bias, out_dtype, out,

@@ -465,12 +465,8 @@ bq_status launch_qskinny(const void* x, int x_dtype, const uint32_t* w, const fl
 #define BQ_SKINNY_F32(V)                                                                             \
   do {                                                                                               \
     auto kernel = qskinny_f32_kernel<V>;                                                             \
-    static bool configured = false;                                                                  \
-    if (!configured && lds > 65536) { /* only the largest slices need the opt-in */                  \
-      BQ_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),                              \
-                                 hipFuncAttributeMaxDynamicSharedMemorySize, 65536 + 256));          \
-      configured = true;                                                                             \
-    }                                                                                                \
+    /* refused on the host when the device grants less; the largest slices need the opt-in */        \
+    BQ_TRY(configure_dynamic_lds(reinterpret_cast<const void*>(kernel), lds, "qskinny_f32_kernel"));  \
     hipLaunchKernelGGL(kernel, grid, tb, lds, st, static_cast<const float*>(x), w, scales, m, k, n,  \
                        nw, block_words_log2, scales_per_row, per_tensor, p.k_per_wg, part);          \
   } while (0)
@@ -487,12 +483,8 @@ bq_status launch_qskinny(const void* x, int x_dtype, const uint32_t* w, const fl
 #define BQ_SKINNY(V, XB)                                                                           \
   do {                                                                                             \
     auto kernel = qskinny_kernel<V, XB>;                                                           \
-    static bool configured = false;                                                                \
-    if (!configured && lds > 65536) { /* only the largest slices need the opt-in */                \
-      BQ_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),                            \
-                                 hipFuncAttributeMaxDynamicSharedMemorySize, 65536 + 2048));       \
-      configured = true;                                                                           \
-    }                                                                                              \
+    /* refused on the host when the device grants less; the largest slices need the opt-in */      \
+    BQ_TRY(configure_dynamic_lds(reinterpret_cast<const void*>(kernel), lds, "qskinny_kernel"));    \
     hipLaunchKernelGGL(kernel, grid, tb, lds, st, x, w, scales, m, k, n, nw, block_words_log2,     \
                        scales_per_row, per_tensor, p.k_per_wg, part);                              \
   } while (0)

@@ -405,13 +405,8 @@ bq_status launch_qsplit(const void* x, int x_dtype, const uint32_t* w, const flo
 #define BQ_SPLIT2(V, PT, XB, T, S)                                                                          \
   do {                                                                                            \
     auto kernel = qsplit_kernel<V, PT, XB, T, S>;                                                           \
-    static bool configured = false;                                                               \
-    if (!configured) { /* the largest slices need more than the default 64 KiB */                 \
-      BQ_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),                           \
-                                 hipFuncAttributeMaxDynamicSharedMemorySize,                      \
-                                 static_cast<int>(16 * T * (kMaxSlice + 4) * sizeof(float) + kSplitWaves * kSlotBytes))); \
-      configured = true;                                                                          \
-    }                                                                                             \
+    /* more than the default 64 KiB: checked against what the device grants, else refused here */ \
+    BQ_TRY(configure_dynamic_lds(reinterpret_cast<const void*>(kernel), lds, "qsplit_kernel"));   \
     hipLaunchKernelGGL(kernel, grid, tb, lds, st, x, w, scales, m, k, n, p.k_per_wg, part);       \
   } while (0)
 #define BQ_SPLIT(V, PT, XB, S)                  \

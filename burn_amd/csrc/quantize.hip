@@ -399,6 +399,37 @@ bq_status launch_fill_u32(uint32_t* dst, size_t n, uint32_t value, hipStream_t s
   return BQ_OK;
 }
 
+// Validate mode: NaNs into counts[0], infinities into counts[1] (one atomic per workgroup that saw any).
+__global__ void __launch_bounds__(256) count_nonfinite_kernel(const float* __restrict__ x, size_t n,
+                                                              uint32_t* __restrict__ counts) {
+  const size_t stride = static_cast<size_t>(gridDim.x) * 256;
+  unsigned nan = 0, inf = 0;
+  for (size_t i = static_cast<size_t>(blockIdx.x) * 256 + threadIdx.x; i < n; i += stride) {
+    const uint32_t mag = __float_as_uint(x[i]) & 0x7FFFFFFFu;
+    nan += mag > 0x7F800000u;
+    inf += mag == 0x7F800000u;
+  }
+  __shared__ unsigned tot[2];
+  if (threadIdx.x == 0) tot[0] = tot[1] = 0;
+  __syncthreads();
+  if (nan) atomicAdd(&tot[0], nan);
+  if (inf) atomicAdd(&tot[1], inf);
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    if (tot[0]) atomicAdd(counts + 0, tot[0]);
+    if (tot[1]) atomicAdd(counts + 1, tot[1]);
+  }
+}
+
+bq_status launch_count_nonfinite(const float* x, size_t n, uint32_t* counts, hipStream_t st) {
+  if (n == 0) return BQ_OK;
+  size_t g = (n + 255) / 256;
+  if (g > 4096) g = 4096;
+  hipLaunchKernelGGL(count_nonfinite_kernel, dim3(static_cast<unsigned>(g)), dim3(256), 0, st, x, n, counts);
+  BQ_HIP(hipGetLastError());
+  return BQ_OK;
+}
+
 // Plain streaming copy, 16 bytes per lane, 4 chunks per workgroup pass: the known-traffic
 // kernel the HBM counters are calibrated against.
 __global__ void __launch_bounds__(256) copy16_kernel(const vuint4* __restrict__ src, vuint4* __restrict__ dst,
@@ -476,11 +507,43 @@ __global__ void selftest_division_kernel(unsigned long long* __restrict__ mismat
   if (bad_4) atomicAdd(mismatches + 2, static_cast<unsigned long long>(bad_4));
 }
 
+// The quotient shortcut x / s (div_by_recip) where a misrounding could change an integer: around
+// every rounding tie. For every scale mantissa (at the lowest, the middle and the highest exponent
+// the shortcut is taken for) and every k in [-128, 127]: x = RN((k + 1/2) * s) and its two
+// neighbours on either side. Counter 3: quotients whose bits differ from the IEEE division;
+// counter 4: quantized integers (clamped to +-127, rounded half away) that differ.
+__global__ void selftest_quotient_kernel(unsigned long long* __restrict__ mismatches) {
+  const uint32_t m = blockIdx.x * blockDim.x + threadIdx.x;
+  if (m >= (1u << 23)) return;
+  unsigned bad_q = 0, bad_i = 0;
+  const uint32_t exps[3] = {27u, 127u, 227u};
+  for (int e = 0; e < 3; ++e) {
+    const float s = __uint_as_float((exps[e] << 23) | m);
+    const float r = recip_exact(s);
+    for (int k = -128; k <= 127; ++k) {
+      const float tie = (static_cast<float>(k) + 0.5f) * s;
+      const uint32_t tb = __float_as_uint(tie);
+#pragma unroll
+      for (int d = -2; d <= 2; ++d) {
+        const float x = __uint_as_float(tb + static_cast<uint32_t>(d));  // neighbours in magnitude
+        const float exact = x / s, fast = div_by_recip(x, s, r);
+        bad_q += __float_as_uint(exact) != __float_as_uint(fast);
+        bad_i += quantize_div(x, s, 127.0f) != quantize_recip(x, s, r, 127.0f);
+      }
+    }
+  }
+  if (bad_q) atomicAdd(mismatches + 3, static_cast<unsigned long long>(bad_q));
+  if (bad_i) atomicAdd(mismatches + 4, static_cast<unsigned long long>(bad_i));
+}
+
 extern "C" bq_status bqk_selftest_division(uint64_t* mismatches_dev, void* stream) {
   BQ_NOTNULL(mismatches_dev);
   hipStream_t st = static_cast<hipStream_t>(stream);
-  BQ_TRY(launch_fill_u32(reinterpret_cast<uint32_t*>(mismatches_dev), 6, 0u, st));
+  BQ_TRY(launch_fill_u32(reinterpret_cast<uint32_t*>(mismatches_dev), 10, 0u, st));
   hipLaunchKernelGGL(selftest_division_kernel, dim3((1u << 23) / 256), dim3(256), 0, st,
+                     reinterpret_cast<unsigned long long*>(mismatches_dev));
+  BQ_HIP(hipGetLastError());
+  hipLaunchKernelGGL(selftest_quotient_kernel, dim3((1u << 23) / 256), dim3(256), 0, st,
                      reinterpret_cast<unsigned long long*>(mismatches_dev));
   BQ_HIP(hipGetLastError());
   return BQ_OK;

@@ -59,7 +59,9 @@ static size_t value_bytes(const bq_scheme& s, const size_t* shape, int rank) {
 }
 
 // What the backend accepts: the same conditions under which the reference backends panic.
-static bq_status check_scheme(const bq_scheme& s, const size_t* shape, int rank) {
+// `storable`: also require what a packed device tensor needs (whole words along the last dim). The
+// length formula alone (quantized_data_len) pads a ragged last dim to whole words instead.
+static bq_status check_scheme(const bq_scheme& s, const size_t* shape, int rank, bool storable = true) {
   if (rank < 1 || rank > BQ_MAX_RANK) BQ_FAIL(BQ_ERR_SHAPE, "rank %d outside 1..%d", rank, BQ_MAX_RANK);
   if (!value_known(s.value))
     BQ_FAIL(BQ_ERR_UNSUPPORTED_SCHEME, "Quantization not supported for value %d (Q8S and Q4S are)", s.value);
@@ -70,7 +72,7 @@ static bq_status check_scheme(const bq_scheme& s, const size_t* shape, int rank)
   if (s.store == BQ_STORE_NATIVE) {
     if (s.value != BQ_Q8S) BQ_FAIL(BQ_ERR_UNSUPPORTED_SCHEME, "Can't store native sub-byte values");
   } else if (s.store == BQ_STORE_PACKED_U32) {
-    if (shape[rank - 1] % static_cast<size_t>(num_quants(s.value)))
+    if (storable && shape[rank - 1] % static_cast<size_t>(num_quants(s.value)))
       BQ_FAIL(BQ_ERR_SHAPE, "Can't store in u32: last dim %zu is not a multiple of %d", shape[rank - 1],
               num_quants(s.value));
   } else {
@@ -110,16 +112,11 @@ long run_block(const bq_scheme& s, const size_t* shape, int rank) {
 using namespace bq;
 
 // ================================================================================ device context
-bq_status bq_device::alloc(size_t bytes, void** out) {
+bq_status bq_device::alloc(size_t bytes, void** out, size_t* actual) {
   bytes = round_up(bytes ? bytes : 1, 512);
   {
     std::lock_guard<std::mutex> lock(mu);
-    auto it = free_blocks.find(bytes);
-    if (it != free_blocks.end()) {
-      *out = it->second;
-      free_blocks.erase(it);
-      return BQ_OK;
-    }
+    if (cache.take(bytes, out, actual)) return BQ_OK;
   }
   BQ_HIP(hipSetDevice(ordinal));
   hipError_t e = hipMalloc(out, bytes);
@@ -128,6 +125,9 @@ bq_status bq_device::alloc(size_t bytes, void** out) {
     BQ_TRY(trim());  // return the cache to the driver and retry once
     BQ_HIP(hipMalloc(out, bytes));
   }
+  *actual = bytes;
+  std::lock_guard<std::mutex> lock(mu);
+  cache.note_handed_out(*out);
   return BQ_OK;
 }
 
@@ -135,29 +135,39 @@ void bq_device::release(void* ptr, size_t bytes) {
   if (!ptr) return;
   std::lock_guard<std::mutex> lock(mu);
   // Reuse is stream ordered: everything that touched this block was enqueued on `stream`
-  // before whatever the next owner enqueues.
-  free_blocks.emplace(round_up(bytes ? bytes : 1, 512), ptr);
+  // before whatever the next owner enqueues. Blocks a HIP graph may still address are parked
+  // with that graph instead (block_cache.hpp).
+  cache.put(ptr, bytes);
 }
 
 bq_status bq_device::trim() {
-  std::multimap<size_t, void*> blocks;
+  std::vector<void*> blocks, retired;
   {
     std::lock_guard<std::mutex> lock(mu);
-    blocks.swap(free_blocks);
+    if (cache.capturing()) BQ_FAIL(BQ_ERR_UNSUPPORTED_OP, "bq_device_trim while the stream is being captured");
+    blocks = cache.drain();
+    retired = cache.take_retired();
   }
-  if (blocks.empty()) return BQ_OK;
+  if (blocks.empty() && retired.empty()) return BQ_OK;
   BQ_HIP(hipSetDevice(ordinal));
   BQ_HIP(hipStreamSynchronize(stream));
-  for (auto& kv : blocks) (void)hipFree(kv.second);
+  for (void* p : blocks) (void)hipFree(p);
+  for (void* p : retired) (void)hipFree(p);
   return BQ_OK;
 }
 
+// Called with `mu` held. A workspace that a captured graph may address is never freed while that
+// graph can still be replayed: it is retired and freed once no graph is left (trim / close).
 bq_status bq_device::ensure_workspace(size_t bytes) {
   if (bytes <= workspace_bytes) return BQ_OK;
   BQ_HIP(hipSetDevice(ordinal));
   if (workspace) {
-    BQ_HIP(hipStreamSynchronize(stream));
-    (void)hipFree(workspace);
+    if (cache.must_retire()) {
+      cache.retire(workspace);  // (no synchronisation either: the stream may be capturing)
+    } else {
+      BQ_HIP(hipStreamSynchronize(stream));
+      (void)hipFree(workspace);
+    }
     workspace = nullptr;
     workspace_bytes = 0;
   }
@@ -166,6 +176,49 @@ bq_status bq_device::ensure_workspace(size_t bytes) {
   workspace_bytes = bytes;
   return BQ_OK;
 }
+
+// ---- dynamic LDS requests ------------------------------------------------------------------------
+namespace bq {
+
+bq_status lds_request_status(size_t bytes, size_t device_limit, const char* what) {
+  if (bytes > device_limit)
+    BQ_FAIL(BQ_ERR_HIP, "%s asks for %zu bytes of LDS, the device grants %zu per workgroup: launch refused",
+            what ? what : "kernel", bytes, device_limit);
+  return BQ_OK;
+}
+
+static size_t device_lds_limit(int ordinal) {
+  static std::mutex mu;
+  static size_t limits[64] = {0};
+  std::lock_guard<std::mutex> lock(mu);
+  if (ordinal < 0 || ordinal >= 64) return 64 * 1024;
+  if (limits[ordinal] == 0) {
+    int plain = 0, optin = 0;
+    if (hipDeviceGetAttribute(&plain, hipDeviceAttributeMaxSharedMemoryPerBlock, ordinal) != hipSuccess) plain = 0;
+    if (hipDeviceGetAttribute(&optin, hipDeviceAttributeSharedMemPerBlockOptin, ordinal) != hipSuccess) optin = 0;
+    (void)hipGetLastError();
+    const int best = std::max(plain, optin);
+    limits[ordinal] = best > 0 ? static_cast<size_t>(best) : 64 * 1024;
+  }
+  return limits[ordinal];
+}
+
+bq_status configure_dynamic_lds(const void* kernel, size_t bytes, const char* what) {
+  int ordinal = 0;
+  BQ_HIP(hipGetDevice(&ordinal));
+  BQ_TRY(lds_request_status(bytes, device_lds_limit(ordinal), what));
+  static std::mutex mu;
+  static std::map<std::pair<int, const void*>, size_t> raised;  // (device, kernel) -> attribute set so far
+  std::lock_guard<std::mutex> lock(mu);
+  size_t& have = raised[std::make_pair(ordinal, kernel)];
+  if (have < bytes) {
+    BQ_HIP(hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(bytes)));
+    have = bytes;
+  }
+  return BQ_OK;
+}
+
+}  // namespace bq
 
 static std::mutex g_devices_mu;
 static bq_device* g_devices[64] = {nullptr};
@@ -205,6 +258,7 @@ extern "C" bq_status bq_device_open(int32_t ordinal, bq_device** out) {
   dev->ordinal = ordinal;
   hipDeviceProp_t prop;
   if (hipGetDeviceProperties(&prop, ordinal) == hipSuccess) dev->num_cus = prop.multiProcessorCount;
+  dev->lds_limit = device_lds_limit(ordinal);
   hipError_t se = hipStreamCreateWithFlags(&dev->stream, hipStreamNonBlocking);
   if (se == hipSuccess) se = hipEventCreate(&dev->ev_start);
   if (se == hipSuccess) se = hipEventCreate(&dev->ev_stop);
@@ -224,6 +278,7 @@ extern "C" bq_status bq_device_close(bq_device* dev) {
   BQ_HIP(hipStreamSynchronize(dev->stream));
   BQ_TRY(dev->trim());
   if (dev->workspace) (void)hipFree(dev->workspace);
+  if (dev->validate_cells) (void)hipFree(dev->validate_cells);
   (void)hipEventDestroy(dev->ev_start);
   (void)hipEventDestroy(dev->ev_stop);
   (void)hipStreamDestroy(dev->stream);
@@ -243,6 +298,16 @@ extern "C" void* bq_device_stream(bq_device* dev) { return dev ? dev->stream : n
 extern "C" bq_status bq_device_trim(bq_device* dev) {
   BQ_NOTNULL(dev);
   return dev->trim();
+}
+
+extern "C" bq_status bq_device_set_validate(bq_device* dev, int32_t on) {
+  BQ_NOTNULL(dev);
+  dev->validate.store(on != 0);
+  return BQ_OK;
+}
+
+extern "C" bq_status bqk_lds_request_status(size_t bytes, size_t device_limit) {
+  return lds_request_status(bytes, device_limit, "kernel");
 }
 
 extern "C" bq_status bq_timer_start(bq_device* dev) {
@@ -265,12 +330,19 @@ struct bq_graph {
   bq_device* dev = nullptr;
   hipGraph_t graph = nullptr;
   hipGraphExec_t exec = nullptr;
+  bq::GraphBlocks blocks;  // allocations the captured kernels address (block_cache.hpp)
 };
 
 extern "C" bq_status bq_graph_begin_capture(bq_device* dev) {
   BQ_NOTNULL(dev);
+  {
+    std::lock_guard<std::mutex> lock(dev->mu);
+    if (dev->cache.capturing()) BQ_FAIL(BQ_ERR_UNSUPPORTED_OP, "a capture is already open on this device");
+  }
   // relaxed: an allocation-cache miss inside the captured region may still call hipMalloc
   BQ_HIP(hipStreamBeginCapture(dev->stream, hipStreamCaptureModeRelaxed));
+  std::lock_guard<std::mutex> lock(dev->mu);
+  dev->cache.begin_capture();
   return BQ_OK;
 }
 
@@ -279,17 +351,26 @@ extern "C" bq_status bq_graph_end_capture(bq_device* dev, bq_graph** out) {
   BQ_NOTNULL(out);
   *out = nullptr;
   hipGraph_t graph = nullptr;
-  BQ_HIP(hipStreamEndCapture(dev->stream, &graph));
+  hipError_t e = hipStreamEndCapture(dev->stream, &graph);
   hipGraphExec_t exec = nullptr;
-  hipError_t e = hipGraphInstantiate(&exec, graph, nullptr, nullptr, 0);
+  if (e == hipSuccess) {
+    e = hipGraphInstantiate(&exec, graph, nullptr, nullptr, 0);
+    if (e != hipSuccess) (void)hipGraphDestroy(graph);
+  }
   if (e != hipSuccess) {
-    (void)hipGraphDestroy(graph);
-    BQ_FAIL(BQ_ERR_HIP, "hipGraphInstantiate failed: %s", hipGetErrorString(e));
+    (void)hipGetLastError();
+    std::lock_guard<std::mutex> lock(dev->mu);
+    dev->cache.end_capture(nullptr);
+    BQ_FAIL(BQ_ERR_HIP, "ending the capture / instantiating the graph failed: %s", hipGetErrorString(e));
   }
   bq_graph* g = new bq_graph();
   g->dev = dev;
   g->graph = graph;
   g->exec = exec;
+  {
+    std::lock_guard<std::mutex> lock(dev->mu);
+    dev->cache.end_capture(&g->blocks);
+  }
   *out = g;
   return BQ_OK;
 }
@@ -302,9 +383,13 @@ extern "C" bq_status bq_graph_launch(bq_graph* g) {
 
 extern "C" bq_status bq_graph_release(bq_graph* g) {
   BQ_NOTNULL(g);
-  (void)hipStreamSynchronize(g->dev->stream);
+  (void)hipStreamSynchronize(g->dev->stream);  // the last replay has finished
   (void)hipGraphExecDestroy(g->exec);
   (void)hipGraphDestroy(g->graph);
+  {
+    std::lock_guard<std::mutex> lock(g->dev->mu);
+    g->dev->cache.release_graph(&g->blocks);
+  }
   delete g;
   return BQ_OK;
 }
@@ -322,8 +407,7 @@ static bq_status new_float(bq_device* dev, int32_t dtype, const size_t* shape, i
   t->rank = rank;
   for (int d = 0; d < rank; ++d) t->shape[d] = shape[d];
   t->value_bytes = t->numel() * dtype_size(dtype);
-  t->alloc_bytes = round_up(t->value_bytes ? t->value_bytes : 1, 512);
-  bq_status s = dev->alloc(t->alloc_bytes, &t->data);
+  bq_status s = dev->alloc(round_up(t->value_bytes ? t->value_bytes : 1, 512), &t->data, &t->alloc_bytes);
   if (s != BQ_OK) {
     delete t;
     return s;
@@ -346,8 +430,8 @@ static bq_status new_quantized(bq_device* dev, const bq_scheme& scheme, const si
   t->value_bytes = value_bytes(scheme, shape, rank);
   t->num_scales = num_params(scheme, shape, rank);
   t->scales_offset = round_up(t->value_bytes, 256);
-  t->alloc_bytes = round_up(t->scales_offset + 4 * (t->num_scales + 1 + BQ_ABSMAX_CELLS), 512);
-  bq_status s = dev->alloc(t->alloc_bytes, &t->data);
+  bq_status s = dev->alloc(round_up(t->scales_offset + 4 * (t->num_scales + 1 + BQ_ABSMAX_CELLS), 512), &t->data,
+                           &t->alloc_bytes);
   if (s != BQ_OK) {
     delete t;
     return s;
@@ -467,8 +551,9 @@ extern "C" bq_status bq_quantized_data_len(const bq_scheme* scheme, const size_t
   BQ_NOTNULL(scheme);
   BQ_NOTNULL(shape);
   BQ_NOTNULL(len_out);
-  if (!value_known(scheme->value)) BQ_FAIL(BQ_ERR_UNSUPPORTED_SCHEME, "unknown quant value %d", scheme->value);
-  if (rank < 1 || rank > BQ_MAX_RANK) BQ_FAIL(BQ_ERR_SHAPE, "rank %d outside 1..%d", rank, BQ_MAX_RANK);
+  // (a zero block extent, a dim the block does not divide, an unknown store or level are refused
+  // here; a ragged last dim is not: the formula pads it to whole words, burn-store's data_len cases)
+  BQ_TRY(check_scheme(*scheme, shape, rank, false));
   *len_out = value_bytes(*scheme, shape, rank) + 4 * num_params(*scheme, shape, rank);
   return BQ_OK;
 }
@@ -521,6 +606,40 @@ extern "C" bq_status bq_q_into_data(const bq_tensor* t, uint8_t* bytes, size_t c
 }
 
 // ================================================================================ quantize
+// Validate mode (bq_device_set_validate): the reference panics when a quotient x / scale is NaN
+// (`Q::from(..).unwrap()`, crates/burn-ndarray/src/ops/quantization.rs:128-133). That happens for a
+// NaN input, a NaN scale, and inf / inf: an infinite input against an infinite scale, which is every
+// infinite input of a quantize_dynamic (its own range makes the scale infinite). The inputs are
+// counted on the device and the call fails before anything is quantized. (With given scales an
+// infinite input and an infinite scale anywhere are refused together, also when they belong to
+// different blocks.) Synchronises the stream: a debugging aid, not for captured or timed loops.
+static bq_status validate_quantize_inputs(bq_device* dev, const float* x, size_t n, const float* scales,
+                                          size_t n_scales) {
+  {
+    std::lock_guard<std::mutex> lock(dev->mu);
+    if (dev->cache.capturing())
+      BQ_FAIL(BQ_ERR_UNSUPPORTED_OP, "the validate mode synchronises the stream and cannot be captured");
+    if (dev->validate_cells == nullptr) {
+      BQ_HIP(hipSetDevice(dev->ordinal));
+      BQ_HIP(hipMalloc(reinterpret_cast<void**>(&dev->validate_cells), 4 * sizeof(uint32_t)));
+    }
+  }
+  hipStream_t st = dev->stream;
+  BQ_TRY(launch_fill_u32(dev->validate_cells, 4, 0u, st));
+  BQ_TRY(launch_count_nonfinite(x, n, dev->validate_cells, st));
+  if (scales != nullptr) BQ_TRY(launch_count_nonfinite(scales, n_scales, dev->validate_cells + 2, st));
+  uint32_t host[4] = {0, 0, 0, 0};
+  BQ_HIP(hipMemcpyAsync(host, dev->validate_cells, sizeof(host), hipMemcpyDeviceToHost, st));
+  BQ_HIP(hipStreamSynchronize(st));
+  const bool dynamic = scales == nullptr;
+  if (host[0] || host[2] || (host[1] && (dynamic || host[3])))
+    BQ_FAIL(BQ_ERR_NONFINITE,
+            "quantize: x / scale is NaN for some element (%u NaN and %u infinite inputs, %u NaN and %u infinite "
+            "scales); the reference panics here",
+            host[0], host[1], host[2], host[3]);
+  return BQ_OK;
+}
+
 static bq_status quantize_impl(const bq_tensor* x, const bq_scheme* scheme, const bq_tensor* scales,
                                bq_tensor** out) {
   BQ_NOTNULL(x);
@@ -532,15 +651,23 @@ static bq_status quantize_impl(const bq_tensor* x, const bq_scheme* scheme, cons
   bq_tensor* q = nullptr;
   BQ_TRY(new_quantized(x->dev, *scheme, x->shape, x->rank, &q));
   if (!dynamic) {
-    if (scales->dtype != BQ_F32 || scales->numel() != q->num_scales) {
+    if (scales->dtype != BQ_F32 || scales->numel() != q->num_scales || scales->dev != x->dev) {
       bq_tensor_release(q);
-      BQ_FAIL(BQ_ERR_SHAPE, "scales must be an f32 tensor of %zu entries", q->num_scales);
+      BQ_FAIL(BQ_ERR_SHAPE, "scales must be an f32 tensor of %zu entries on the input's device", q->num_scales);
     }
   }
   hipStream_t st = x->dev->stream;
   const size_t n = x->numel();
   const float* xin = static_cast<const float*>(x->data);
   bq_status rc = BQ_OK;
+  if (x->dev->validate.load()) {
+    rc = validate_quantize_inputs(x->dev, xin, n, dynamic ? nullptr : static_cast<const float*>(scales->data),
+                                  dynamic ? 0 : q->num_scales);
+    if (rc != BQ_OK) {
+      bq_tensor_release(q);
+      return rc;
+    }
+  }
   do {
     if (!dynamic) {
       hipError_t e = hipMemcpyAsync(q->scales(), scales->data, 4 * q->num_scales, hipMemcpyDeviceToDevice, st);
@@ -678,6 +805,7 @@ extern "C" bq_status bq_float_matmul(const bq_tensor* lhs, const bq_tensor* rhs,
   BQ_NOTNULL(rhs);
   BQ_NOTNULL(out);
   if (lhs->dtype == BQ_QFLOAT || rhs->dtype == BQ_QFLOAT) BQ_FAIL(BQ_ERR_DTYPE, "float_matmul takes float tensors");
+  if (lhs->dev != rhs->dev) BQ_FAIL(BQ_ERR_DTYPE, "float_matmul operands live on different devices");
   MatmulDims d;
   BQ_TRY(matmul_dims(lhs, rhs, &d));
   bq_tensor* o = nullptr;
@@ -714,6 +842,7 @@ static bq_status q_matmul_impl(const bq_tensor* lhs, const bq_tensor* rhs, int32
   MatmulDims d;
   BQ_TRY(matmul_dims(lhs, rhs, &d));
   bq_device* dev = lhs->dev;
+  if (rhs->dev != dev) BQ_FAIL(BQ_ERR_DTYPE, "q_matmul operands live on different devices (%d and %d)", dev->ordinal, rhs->dev->ordinal);
   hipStream_t st = dev->stream;
 
   // Fused path: float lhs x quantized rhs whose scales are per tensor or runs along N.
@@ -855,6 +984,8 @@ extern "C" bq_status bq_q_linear(const bq_tensor* x, const bq_tensor* weight, co
     BQ_FAIL(BQ_ERR_DTYPE, "out dtype must be f32 or bf16");
   const size_t d_in = weight->shape[0], d_out = weight->shape[1];
   bq_device* dev = x->dev;
+  if (weight->dev != dev || (bias != nullptr && bias->dev != dev))
+    BQ_FAIL(BQ_ERR_DTYPE, "q_linear operands live on different devices");
   bq_tensor* bias32 = nullptr;  // f32 copy of a bf16 bias
   const float* bias_ptr = nullptr;
   if (bias != nullptr) {

@@ -44,6 +44,11 @@ class Device:
     def trim(self):
         check(lib().bq_device_trim(self.handle))
 
+    def set_validate(self, on: bool):
+        """Validate mode: quantize fails with ERR_NONFINITE where the reference panics on a NaN
+        quotient (NaN input or scale, infinite input against an infinite scale)."""
+        check(lib().bq_device_set_validate(self.handle, 1 if on else 0))
+
     @property
     def stream(self) -> int:
         return lib().bq_device_stream(self.handle) or 0

@@ -44,7 +44,8 @@ enum {
   BQ_ERR_DTYPE = 4,              /* float/quantized mix-up or unsupported float dtype */
   BQ_ERR_HIP = 5,                /* a HIP runtime call failed (ExecutionError on the Rust side) */
   BQ_ERR_SIZE = 6,               /* host buffer too small / blob shorter than its scheme requires */
-  BQ_ERR_UNSUPPORTED_OP = 7      /* layout op this backend declines (reference: unimplemented!()) */
+  BQ_ERR_UNSUPPORTED_OP = 7,     /* layout op this backend declines (reference: unimplemented!()) */
+  BQ_ERR_NONFINITE = 8           /* validate mode: x / scale is NaN (reference: Q::from(NaN).unwrap() panics) */
 };
 
 /* DType of a handle. BQ_QFLOAT carries a bq_scheme, like DType::QFloat(scheme). */
@@ -89,6 +90,15 @@ bq_status bq_device_sync(bq_device* dev);
 void* bq_device_stream(bq_device* dev);
 /* Returns cached, currently unused device allocations to the driver. */
 bq_status bq_device_trim(bq_device* dev);
+/* Validate mode (off by default). While on, bq_quantize / bq_quantize_dynamic first count the
+ * NaN and infinite inputs (and scales) on the device and fail with BQ_ERR_NONFINITE where the
+ * reference panics: a quotient x / scale that is NaN cannot become an integer
+ * (crates/burn-ndarray/src/ops/quantization.rs:128-133, `Q::from(..).unwrap()`). That is a NaN input
+ * or scale, or an infinite input against an infinite scale -- which includes every infinite input
+ * of a quantize_dynamic, whose own range makes the scale infinite. The check synchronises the
+ * stream (a debugging aid; refused during graph capture). Off, such inputs give unspecified
+ * integers. */
+bq_status bq_device_set_validate(bq_device* dev, int32_t on);
 /* HIP-event stopwatch on the context's stream (what Backend::sync-bracketed benches measure,
  * without the host round trip): start, enqueue work, stop -> elapsed milliseconds. */
 bq_status bq_timer_start(bq_device* dev);
@@ -102,7 +112,14 @@ bq_status bq_timer_stop(bq_device* dev, float* elapsed_ms);
  * cache and the split-K workspace exist), make no *_into_data / *_from_data / sync / timer call
  * while capturing, and keep every tensor created during capture alive for as long as the graph is
  * replayed (their memory is baked into it). The kernels clear their scratch with fill kernels,
- * never memset nodes. */
+ * never memset nodes.
+ * What the library allocates for itself stays valid for the graph's lifetime: temporaries created
+ * and released inside a captured call (the f32 copy of a bf16 bias, dequantized operands of the
+ * general q_matmul path), tensors created during the capture and released afterwards, and the
+ * split-K workspace (a larger one requested later does not free the one a graph addresses) all
+ * return to the allocator only at bq_graph_release. Tensors that existed before the capture and
+ * are read by it are the caller's to keep alive, with their contents. One capture per device at a
+ * time; bq_device_trim is refused while one is open. */
 typedef struct bq_graph bq_graph;
 bq_status bq_graph_begin_capture(bq_device* dev);
 bq_status bq_graph_end_capture(bq_device* dev, bq_graph** out);
@@ -213,16 +230,25 @@ bq_status bq_q_flip(const bq_tensor* t, const int32_t* axes, int32_t n_axes, bq_
 
 /* No counterpart in the reference: a hardware self-check. The quantize kernels replace the IEEE
  * divisions of the reference arithmetic (x / s, 1 / s, (2*amax) / (b-a)) by reciprocal + fma
- * correction sequences that are exact; this launches an exhaustive comparison (all 2^23
- * mantissas x every exponent each shortcut is used for) on the device and leaves three
- * mismatch counts -- reciprocal, Q8S scale, Q4S scale -- in mismatches_dev[0..2] (device memory,
- * 3 x u64). All three must read 0. */
+ * correction sequences that are exact; this launches exhaustive comparisons on the device and
+ * leaves five mismatch counts in mismatches_dev[0..4] (device memory, 5 x u64):
+ *   [0] reciprocal 1 / s, [1] Q8S scale, [2] Q4S scale: all 2^23 mantissas x every exponent the
+ *       shortcut is used for;
+ *   [3] quotient x / s, bit for bit, and [4] the integer it quantizes to: all 2^23 scale mantissas
+ *       (lowest, middle and highest exponent of the shortcut) x every rounding tie (k + 1/2) * s,
+ *       k in [-128, 127], with two neighbours of x on either side.
+ * All five must read 0. */
 bq_status bqk_selftest_division(uint64_t* mismatches_dev, void* stream);
 /* No counterpart in the reference: a plain device-to-device streaming copy of `bytes` bytes
  * (16-byte aligned, multiple of 16). It is the kernel of known traffic that the HBM byte
  * counters of a profile are calibrated against, and the practical ceiling the streaming
  * kernels are compared with. */
 bq_status bqk_copy(const void* src, void* dst, size_t bytes, void* stream);
+/* No counterpart in the reference: the host-side check every kernel with a dynamic LDS request
+ * goes through before it is launched. BQ_ERR_HIP when `bytes` exceeds `device_limit` (the launch
+ * is refused; an over-sized request must never reach the GPU), BQ_OK otherwise. Exported so the
+ * rule can be tested without a GPU. */
+bq_status bqk_lds_request_status(size_t bytes, size_t device_limit);
 /* max |x| over n floats, as BQ_ABSMAX_CELLS partial maxima (bit patterns of non-negative f32):
  * every cell of absmax_cells[0 .. BQ_ABSMAX_CELLS) is written, none needs initialising, and the
  * result is the largest cell (one cell per workgroup, so no atomics).

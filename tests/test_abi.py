@@ -67,6 +67,56 @@ def test_kernel_level_argument_validation_needs_no_gpu():
     assert L.bqk_q_matmul_workspace(2048, 4096, 14336, _lib.BF16, _lib.Q4S) == 0
 
 
+def test_oversized_lds_request_is_refused_on_the_host():
+    """Every kernel with a dynamic LDS request passes this guard before it is launched: a request
+    beyond what the device grants per workgroup is an error on the host, never a launch."""
+    L = _lib.lib()
+    limit = 160 * 1024
+    assert L.bqk_lds_request_status(limit, limit) == _lib.OK
+    assert L.bqk_lds_request_status(64 * 1024, limit) == _lib.OK
+    assert L.bqk_lds_request_status(limit + 512, limit) == _lib.ERR_HIP
+    assert b"launch refused" in L.bq_last_error()
+    assert L.bqk_lds_request_status(64 * 1024 + 1, 64 * 1024) == _lib.ERR_HIP
+
+
+def test_data_len_refuses_what_q_from_data_would_refuse():
+    """quantized_data_len runs the full scheme check: no division by a zero block extent, no
+    length for a shape the scheme cannot hold."""
+    L = _lib.lib()
+    out = C.c_size_t()
+
+    def status(scheme, shape):
+        arr = (C.c_size_t * len(shape))(*shape)
+        c = scheme.to_c() if isinstance(scheme, QuantScheme) else scheme
+        return L.bq_quantized_data_len(C.byref(c), arr, len(shape), C.byref(out))
+
+    assert status(QuantScheme().per_block((32,)), (4, 64)) == _lib.OK and out.value == 256 + 4 * 8
+    zero = QuantScheme().per_block((32,)).to_c()
+    zero.block[0] = 0
+    assert status(zero, (4, 64)) == _lib.ERR_SHAPE
+    assert status(QuantScheme().per_block((32,)), (4, 48)) == _lib.ERR_SHAPE          # 48 % 32
+    assert status(QuantScheme(value=QuantValue.Q4S), (3, 5)) == _lib.OK and out.value == 3 * 4 + 4  # padded words
+    assert status(QuantScheme().per_block((2, 2, 32)), (4, 64)) == _lib.ERR_SHAPE      # block rank > rank
+    bad = QuantScheme().to_c()
+    bad.store = 9
+    assert status(bad, (4, 64)) == _lib.ERR_UNSUPPORTED_SCHEME
+    bad = QuantScheme().to_c()
+    bad.level = 5
+    assert status(bad, (4, 64)) == _lib.ERR_UNSUPPORTED_SCHEME
+
+
+def test_block_cache_rules(tmp_path):
+    """The allocation cache's graph-capture bookkeeping (which released block may be reused
+    when) is plain C++ with no HIP call: compiled and run on the CPU."""
+    import subprocess
+    exe = tmp_path / "test_block_cache"
+    src = os.path.join(ROOT, "tests", "cpp", "test_block_cache.cpp")
+    subprocess.run(["g++", "-std=c++17", "-O1", "-Wall", "-I", os.path.join(ROOT, "burn_amd", "csrc"), src,
+                    "-o", str(exe)], check=True)
+    out = subprocess.run([str(exe)], check=True, capture_output=True, text=True).stdout
+    assert "block cache: ok" in out
+
+
 def test_no_cpu_fallback():
     if ba.Device.count() > 0:
         pytest.skip("a GPU is present")

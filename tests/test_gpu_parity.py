@@ -184,13 +184,15 @@ def test_scale_exponent_sweep(dev, value):
 
 
 def test_division_shortcuts_are_exact_on_this_gpu(dev):
-    """The kernels replace IEEE divisions by reciprocal + fma sequences; the library can compare
-    the two exhaustively (2^23 mantissas x every admitted exponent) on the device."""
+    """The kernels replace IEEE divisions by reciprocal + fma sequences; the library compares the
+    two exhaustively on the device: 1 / s and the two scale formulas over 2^23 mantissas x every
+    admitted exponent, and the quotient x / s (bits, and the integer it rounds to) around every
+    rounding tie (k + 1/2) * s for every scale mantissa."""
     from burn_amd import _lib
-    buf = FloatOps.float_empty((8,), dev)
+    buf = FloatOps.float_empty((16,), dev)
     _lib.check(_lib.lib().bqk_selftest_division(buf.data_ptr, dev.stream))
-    counts = FloatOps.float_into_data(buf).view(np.uint64)[:3]
-    assert counts.tolist() == [0, 0, 0], counts
+    counts = FloatOps.float_into_data(buf).view(np.uint64)[:5]
+    assert counts.tolist() == [0, 0, 0, 0, 0], counts
 
 
 def test_copy_kernel(dev):
@@ -494,6 +496,89 @@ def test_hip_graph_replays_match_eager(dev):
         dev.sync()
 
 
+def test_hip_graph_keeps_the_librarys_own_buffers(dev):
+    """A captured call that allocates and frees inside itself (the f32 copy of a bf16 bias, the
+    dequantized operands of the general q_matmul path, the float product of a propagating
+    q_matmul) and a workspace that grows after the capture: neither may be recycled while the
+    graph can be replayed. Bystander tensors allocated between replays keep their contents and
+    every replay gives the eager result."""
+    from burn_amd import ModuleOps
+    rng = np.random.default_rng(77)
+    w = QTensorOps.quantize_dynamic(FloatOps.float_from_data(awkward((512, 256), 2), dev), QuantScheme().per_block((32,)))
+    wq_lhs = QTensorOps.quantize_dynamic(FloatOps.float_from_data(awkward((48, 512), 3), dev), QuantScheme().per_block((32,)))
+    a16 = FloatOps.float_from_data(rng.standard_normal((16, 512)).astype(np.float32), dev)
+    bias_bf16 = FloatOps.float_from_data(ba.bf16_bits_from_f32(rng.standard_normal(256).astype(np.float32)), dev, ba.BF16)
+
+    def step():
+        return (ModuleOps.linear(a16, w, bias_bf16),          # temporary: f32 copy of the bias
+                QTensorOps.q_matmul(wq_lhs, w),                # temporaries: both operands dequantized
+                QTensorOps.q_matmul_propagate(a16, w))         # temporary: the float product
+
+    def snapshot(ts):
+        return [QTensorOps.q_into_data(t).bytes.tobytes() if t.is_quantized
+                else FloatOps.float_into_data(t).tobytes() for t in ts]
+
+    eager = snapshot(step())
+    graph, outs = dev.capture(step)
+    bystanders = []
+    for i in range(4):
+        # eager allocations of the temporaries' sizes: they must not land on memory the graph writes
+        fill = np.full(256, float(i + 1), np.float32)
+        mine = [FloatOps.float_from_data(fill, dev) for _ in range(6)]
+        mine += [FloatOps.float_from_data(np.full((48, 512), float(i + 1), np.float32), dev),
+                 FloatOps.float_from_data(np.full((512, 256), float(i + 1), np.float32), dev),
+                 FloatOps.float_from_data(np.full((16, 256), float(i + 1), np.float32), dev)]
+        bystanders.append((i + 1, mine))
+        if i == 1:  # a larger split-K workspace than the captured calls used
+            big = QTensorOps.quantize_dynamic(FloatOps.float_from_data(awkward((2048, 4096), 9), dev),
+                                              QuantScheme().per_block((32,)))
+            a8 = FloatOps.float_from_data(rng.standard_normal((16, 2048)).astype(np.float32), dev)
+            FloatOps.float_into_data(QTensorOps.q_matmul(a8, big))
+        graph.launch()
+        dev.sync()
+        assert snapshot(outs) == eager, f"replay {i} differs from the eager result"
+        for value, tensors in bystanders:
+            for t in tensors:
+                assert (FloatOps.float_into_data(t) == value).all(), "a replay wrote into a bystander tensor"
+    del graph
+    # once the graph is gone its parked blocks are reusable and still intact as allocations
+    again = snapshot(step())
+    assert again == eager
+
+
+def test_validate_mode_fails_where_the_reference_panics(dev):
+    """NaN quotients: the reference panics (Q::from(NaN).unwrap()); in validate mode the call
+    fails with ERR_NONFINITE, out of it the call goes through."""
+    from burn_amd import _lib
+    x = awkward((8, 64), 5)
+    bad_nan, bad_inf = x.copy(), x.copy()
+    bad_nan[3, 7] = np.nan
+    bad_inf[2, 9] = np.inf
+    scheme = QuantScheme().per_block((32,))
+    ok_scales = FloatOps.float_from_data(np.full(16, 0.05, np.float32), dev)
+    inf_scales = FloatOps.float_from_data(np.float32([0.05] * 15 + [np.inf]), dev)
+    nan_scales = FloatOps.float_from_data(np.float32([0.05] * 15 + [np.nan]), dev)
+    dev.set_validate(True)
+    try:
+        QTensorOps.quantize_dynamic(FloatOps.float_from_data(x, dev), scheme)             # finite: fine
+        QTensorOps.quantize(FloatOps.float_from_data(bad_inf, dev), scheme, ok_scales)    # inf / finite clamps
+        QTensorOps.quantize(FloatOps.float_from_data(x, dev), scheme, inf_scales)         # finite / inf = 0
+        for tensor, scales in ((bad_nan, None), (bad_inf, None), (bad_nan, ok_scales), (x, nan_scales),
+                               (bad_inf, inf_scales)):
+            with pytest.raises(ba.BurnqError) as e:
+                t = FloatOps.float_from_data(tensor, dev)
+                if scales is None:
+                    QTensorOps.quantize_dynamic(t, scheme)
+                    QTensorOps.quantize_dynamic(t, QuantScheme(store=QuantStore.Native))
+                else:
+                    QTensorOps.quantize(t, scheme, scales)
+            assert e.value.status == _lib.ERR_NONFINITE
+    finally:
+        dev.set_validate(False)
+    QTensorOps.quantize_dynamic(FloatOps.float_from_data(bad_nan, dev), scheme)  # unspecified integers, no error
+    dev.sync()
+
+
 # ------------------------------------------------------------------ the configs at full size
 
 def test_config1_per_tensor_q8s_native_4096(dev):
@@ -529,16 +614,13 @@ def test_config3_q4s_block32_dequantize_14336x4096(dev):
     assert gblob.bytes.tobytes() == blob.tobytes()
 
 
-def matmul_check(out, ref64, elementwise_all=True):
-    """max |y - y'| / max |y'| <= 1e-2, and burn's permissive elementwise rule: for every element,
-    or (bf16 operands, tens of millions of outputs) for all but a 1e-5 fraction."""
+def matmul_check(out, ref64, max_outside=0):
+    """max |y - y'| / max |y'| <= 1e-2, and burn's permissive elementwise rule for every element
+    (all but `max_outside`, a literal count the caller justifies)."""
     rel = np.abs(out - ref64).max() / np.abs(ref64).max()
     assert rel <= 1e-2, rel
     ok = burn_approx_eq(out, ref64, 1e-2, 1e-2)
-    if elementwise_all:
-        assert ok.all(), f"{(~ok).sum()} outside burn's permissive tolerance"
-    else:
-        assert (~ok).mean() <= 1e-5, f"{(~ok).sum()} of {ok.size} outside burn's permissive tolerance"
+    assert (~ok).sum() <= max_outside, f"{(~ok).sum()} of {ok.size} outside burn's permissive tolerance"
     return rel
 
 
@@ -566,6 +648,19 @@ def test_config4_decode_qgemv(dev, weights_q8, m):
     assert FloatOps.float_into_data(out2).tobytes() == FloatOps.float_into_data(out).tobytes()
 
 
+# C5 against the f32 reference, burn's elementwise rule |y - y'| < max(1e-2 * max(|y|, |y'|), 1e-2):
+# the weights reach the MFMA as bf16(s * q), a relative rounding error of at most 2^-8 (rms about
+# 1.6e-3) per weight. An output sums 4096 products of N(0,1) activations and N(0, 0.02^2) weights
+# (sum of squares 1.64), so its error is close to normal with sigma 1.28 * 1.6e-3 = 2.1e-3 (measured
+# rms 2.126e-3, max 1.25e-2). The rule's 1e-2 floor is 4.70 sigma away: 29 360 128 outputs x
+# P(|z| > 4.70) = 2.6e-6 predicts 76 outputs outside it; 52 are measured (the inputs are seeded and
+# the kernel's summation order is fixed, so the count is reproducible). More than 100 would mean
+# an error that the weight rounding does not explain; the sampled rows (688 128 outputs, 1
+# measured) may hold 5.
+C5_MAX_OUTSIDE = 100
+C5_MAX_OUTSIDE_SAMPLE = 5
+
+
 def test_config5_prefill_qgemm_bf16_q4s(dev):
     rng = np.random.default_rng(0xC5)
     w = (rng.standard_normal((4096, 14336)) * 0.02).astype(np.float32)
@@ -578,14 +673,15 @@ def test_config5_prefill_qgemm_bf16_q4s(dev):
     assert out.shape == (2048, 14336) and out.dtype == ba.F32
     got = FloatOps.float_into_data(out)
     wd = co.dequantize(q_ref, oscheme(scheme), s_ref, mt=True)
-    # float64 yardstick on a sample of rows, f32 sgemm on everything
-    # float64 yardstick on a sample of rows, f32 sgemm on everything. The weights reach the MFMA
-    # as bf16(s * q): that rounding (2^-9 relative per weight) is the whole error budget, about
-    # 2e-3 absolute per output here, so a handful of 29 M outputs near zero can exceed the 1e-2
-    # absolute floor of the elementwise rule while max-relative error stays near 2e-3.
+    # float64 yardstick on a sample of rows, f32 sgemm on everything (see C5_MAX_OUTSIDE above)
     rows = rng.choice(2048, 48, replace=False)
-    matmul_check(got[rows], a[rows].astype(np.float64) @ wd.astype(np.float64), elementwise_all=False)
-    matmul_check(got, (a @ wd).astype(np.float64), elementwise_all=False)
+    ref32 = (a @ wd).astype(np.float64)
+    err = np.abs(got - ref32)
+    outside = int((~burn_approx_eq(got, ref32, 1e-2, 1e-2)).sum())
+    print(f"C5 elementwise: max |err| {err.max():.3e}, rms {np.sqrt((err ** 2).mean()):.3e}, "
+          f"outside burn's permissive rule: {outside} of {got.size}")
+    matmul_check(got[rows], a[rows].astype(np.float64) @ wd.astype(np.float64), max_outside=C5_MAX_OUTSIDE_SAMPLE)
+    matmul_check(got, ref32, max_outside=C5_MAX_OUTSIDE)
     # against the product with the weights rounded the way the kernel rounds them, the kernel is
     # exact to f32 accumulation error
     wb = ba.f32_from_bf16_bits(ba.bf16_bits_from_f32(wd)).reshape(wd.shape).astype(np.float64)
