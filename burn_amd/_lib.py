@@ -106,7 +106,9 @@ SIGNATURES = {
                             _sz, _vp]),
     "bqk_q_linear": (_i32, [_vp, _i32, _sz, _sz, _sz, _vp, _vp, _i32, _i32, _i32, _vp, _i32, _vp, _vp,
                             _sz, _vp]),
+    "bqk_q_linear_static": (_i32, [_vp, _i32, _sz, _sz, _sz, _vp, _vp, _i32, _i32, _i32, _vp, _i32, _vp, _vp]),
 }
+STATIC_SCRATCH_BYTES = 16 << 20
 
 _lib = None
 

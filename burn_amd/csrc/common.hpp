@@ -160,6 +160,10 @@ bq_status launch_fill_u32(uint32_t* dst, size_t n, uint32_t value, hipStream_t s
 bq_status lds_request_status(size_t bytes, size_t device_limit, const char* what);
 bq_status configure_dynamic_lds(const void* kernel, size_t bytes, const char* what);
 
+// Device address of the static scratch array of bqk_q_linear_static on the current device
+// (qmatmul.hip): resolved once per device.
+bq_status static_scratch_ptr(void** out);
+
 // Counts, over n floats, NaNs into counts[0] and infinities into counts[1] (device u32 cells that
 // the kernel adds to; quantize.hip). Used by the validate mode.
 bq_status launch_count_nonfinite(const float* x, size_t n, uint32_t* counts, hipStream_t stream);

@@ -760,3 +760,56 @@ extern "C" bq_status bqk_q_linear(const void* x, int32_t x_dtype, size_t m, size
   return q_matmul_core(x, x_dtype, m, k, n, w_values, w_scales, block, value, store, bias, out_dtype, out,
                        workspace, workspace_bytes, stream);
 }
+
+// ================================================================================ no allocation
+// bqk_q_linear for callers that cannot allocate (code under HIP graph capture, serving loops,
+// harnesses that forbid hipMalloc): the split-K partials and the bf16 copy of an f32 lhs, which
+// bqk_q_linear takes through its `workspace` argument, live in this file-scope device array
+// instead. Every GPU the library runs on holds its own copy of the array at its own address
+// until the process ends; the address is looked up once per device and the kernels only ever see
+// that pointer (the array's name is a host-side stand-in, not a device address).
+static __device__ __align__(256) unsigned char scratch[BQK_STATIC_SCRATCH_BYTES];
+
+namespace bq {
+
+// The device address of `scratch` on the current device (looked up on first use, then cached).
+bq_status static_scratch_ptr(void** out) {
+  static std::mutex mu;
+  static void* ptrs[64] = {nullptr};
+  int ordinal = 0;
+  BQ_HIP(hipGetDevice(&ordinal));
+  if (ordinal < 0 || ordinal >= 64) BQ_FAIL(BQ_ERR_HIP, "device ordinal %d out of range", ordinal);
+  std::lock_guard<std::mutex> lock(mu);
+  if (ptrs[ordinal] == nullptr) {
+    void* p = nullptr;
+    BQ_HIP(hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)));
+    if (p == nullptr || (reinterpret_cast<uintptr_t>(p) & 255u))
+      BQ_FAIL(BQ_ERR_HIP, "the static scratch array resolved to %p", p);
+    ptrs[ordinal] = p;
+  }
+  *out = ptrs[ordinal];
+  return BQ_OK;
+}
+
+}  // namespace bq
+
+extern "C" bq_status bqk_q_linear_static(const void* x, int32_t x_dtype, size_t m, size_t k, size_t n,
+                                         const void* w_values, const float* w_scales, int32_t block,
+                                         int32_t value, int32_t store, const float* bias, int32_t out_dtype,
+                                         void* out, void* stream) {
+  if (bias != nullptr && (reinterpret_cast<uintptr_t>(bias) & 15u))
+    BQ_FAIL(BQ_ERR_SHAPE, "q_linear bias must be 16-byte aligned");
+  // dry run first: the kernel this product takes and the scratch it uses, before anything is launched
+  size_t need = 0;
+  BQ_TRY(q_matmul_core(x, x_dtype, m, k, n, w_values, w_scales, block, value, store, bias, out_dtype, out, nullptr, 0,
+                       stream, &need));
+  if (need > BQK_STATIC_SCRATCH_BYTES)
+    BQ_FAIL(BQ_ERR_SIZE,
+            "bqk_q_linear_static: this product needs %zu bytes of scratch, the static array holds %zu; "
+            "use bqk_q_linear with a workspace",
+            need, static_cast<size_t>(BQK_STATIC_SCRATCH_BYTES));
+  void* ws = nullptr;
+  BQ_TRY(static_scratch_ptr(&ws));
+  return q_matmul_core(x, x_dtype, m, k, n, w_values, w_scales, block, value, store, bias, out_dtype, out, ws,
+                       BQK_STATIC_SCRATCH_BYTES, stream);
+}

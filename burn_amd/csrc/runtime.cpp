@@ -259,6 +259,13 @@ extern "C" bq_status bq_device_open(int32_t ordinal, bq_device** out) {
   hipDeviceProp_t prop;
   if (hipGetDeviceProperties(&prop, ordinal) == hipSuccess) dev->num_cus = prop.multiProcessorCount;
   dev->lds_limit = device_lds_limit(ordinal);
+  {  // set-up of the allocation-free entry point: this device's address of its static scratch array
+    void* scratch_ptr = nullptr;
+    if (static_scratch_ptr(&scratch_ptr) != BQ_OK) {
+      delete dev;
+      return BQ_ERR_HIP;
+    }
+  }
   hipError_t se = hipStreamCreateWithFlags(&dev->stream, hipStreamNonBlocking);
   if (se == hipSuccess) se = hipEventCreate(&dev->ev_start);
   if (se == hipSuccess) se = hipEventCreate(&dev->ev_stop);

@@ -299,6 +299,23 @@ bq_status bqk_q_linear(const void* x, int32_t x_dtype, size_t m, size_t k, size_
                        int32_t store, const float* bias, int32_t out_dtype, void* out, void* workspace,
                        size_t workspace_bytes, void* stream);
 
+/* No counterpart in the reference: bqk_q_linear for callers that cannot allocate or bring a
+ * workspace -- code under HIP graph capture, tight serving loops, harnesses that forbid hipMalloc.
+ * Same arguments and same results (bit for bit: the same kernels in the same order) as
+ * bqk_q_linear, minus the workspace: split-K partials and the bf16 copy of an f32 lhs go to a
+ * static device array of BQK_STATIC_SCRATCH_BYTES that each GPU the library runs on holds until
+ * the process ends. A product whose kernel needs more scratch than that is refused with
+ * BQ_ERR_SIZE before anything is launched (16 MiB holds the partials of the decode and small-batch
+ * kernels, M <= 32, on a [4096, 14336] weight; the need never exceeds bqk_q_matmul_workspace()).
+ * The call allocates nothing (no hipMalloc / hipFree); the array's device address is looked up
+ * once per device, at bq_device_open or at the first call on that device. All calls on one GPU
+ * share the array: calls that overlap there (different streams or threads) race; calls on one
+ * stream are ordered and need no clearing between them (every cell a call reads it has written). */
+#define BQK_STATIC_SCRATCH_BYTES (16u << 20)
+bq_status bqk_q_linear_static(const void* x, int32_t x_dtype, size_t m, size_t k, size_t n,
+                              const void* w_values, const float* w_scales, int32_t block, int32_t value,
+                              int32_t store, const float* bias, int32_t out_dtype, void* out, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -105,6 +105,21 @@ def test_data_len_refuses_what_q_from_data_would_refuse():
     assert status(bad, (4, 64)) == _lib.ERR_UNSUPPORTED_SCHEME
 
 
+def test_static_scratch_entry_point_refuses_large_products_without_a_gpu():
+    """bqk_q_linear_static checks the scratch it would need against the static array before
+    anything else happens."""
+    L = _lib.lib()
+    buf = np.zeros(64, np.float32)
+    p = buf.ctypes.data
+    buf16 = np.zeros(64 + 4, np.float32)
+    p = (buf16.ctypes.data + 15) & ~15   # the entry points check 16-byte alignment first
+    need = L.bqk_q_matmul_workspace(128, 4096, 14336, _lib.F32, _lib.Q4S)
+    assert need > _lib.STATIC_SCRATCH_BYTES
+    rc = L.bqk_q_linear_static(p, _lib.F32, 128, 4096, 14336, p, p, 32, _lib.Q4S, _lib.STORE_PACKED_U32, None,
+                               _lib.F32, p, None)
+    assert rc == _lib.ERR_SIZE and b"static array holds" in L.bq_last_error(), L.bq_last_error()
+
+
 def test_block_cache_rules(tmp_path):
     """The allocation cache's graph-capture bookkeeping (which released block may be reused
     when) is plain C++ with no HIP call: compiled and run on the CPU."""
