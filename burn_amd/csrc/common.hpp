@@ -111,8 +111,20 @@ long run_block(const bq_scheme& scheme, const size_t* shape, int rank);
 
 // Generic rectangle-block kernels (any block shape): slow, complete.
 bq_status launch_quantize_rect(const float* x, const size_t* shape, int rank, const size_t* blk,
-                               int value, int store, bool dynamic, void* values, float* scales,
+                               int value, int store, bool dynamic, int scale_dtype, void* values, float* scales,
                                hipStream_t stream);
+// Fused quantize kernels with the scheme's scale dtype (quantize.hip). Per tensor: `scale_or_cells`
+// is the scale, or (from_absmax) the absmax cells of pass 1, the derived scale then goes to
+// scale_out. Run blocks: scales_in null = dynamic (scales_out receives them).
+bq_status launch_quantize_per_tensor(const float* x, size_t n, const float* scale_or_cells, bool from_absmax,
+                                     float* scale_out, int value, int store, void* values, int scale_dtype,
+                                     hipStream_t stream);
+bq_status launch_quantize_run_block(const float* x, size_t n, int block, const float* scales_in, float* scales_out,
+                                    int value, int store, void* values, int scale_dtype, hipStream_t stream);
+// dst[i] = scale_to_dtype(src[i]); f32 scales <-> their 2-byte wire form (f16 / bf16).
+bq_status launch_round_scales(const float* src, float* dst, size_t n, int scale_dtype, hipStream_t stream);
+bq_status launch_scales_to_wire(const float* src, void* dst, size_t n, int scale_dtype, hipStream_t stream);
+bq_status launch_scales_from_wire(const void* src, float* dst, size_t n, int scale_dtype, hipStream_t stream);
 bq_status launch_dequantize_rect(const void* values, const size_t* shape, int rank,
                                  const size_t* blk, const float* scales, int value, int store,
                                  int out_dtype, void* out, hipStream_t stream);

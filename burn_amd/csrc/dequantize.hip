@@ -12,7 +12,13 @@ bool fused_block_ok(int block, int value);
 
 namespace {
 
-constexpr int kThreads = 256;
+#ifndef BQ_DEQUANT_THREADS
+#define BQ_DEQUANT_THREADS 256
+#endif
+#ifndef BQ_DEQUANT_UNROLL
+#define BQ_DEQUANT_UNROLL 2
+#endif
+constexpr int kThreads = BQ_DEQUANT_THREADS;
 
 // One lane-step produces one output "chunk": VPC consecutive values stored as a single vector
 // (f32: 4 values = 16 B; bf16: a whole word's 4 or 8 values = 8 or 16 B), so every store
@@ -42,7 +48,7 @@ __device__ __forceinline__ void store_chunk(void* __restrict__ out, size_t chunk
 
 // A workgroup owns kThreads * U consecutive chunks; lane t takes chunks t, t + 256, ...
 // block_words_log2 = log2(words per scale) for run-block schemes.
-constexpr int kDequantUnroll = 2;  // measured on C2 / C1 / C3: 1 -> 60.9 / 17.9 / 49.4 us, 2 -> 53.7 / 16.1 / 47.5, 4 -> 57.3 / 16.4 / 48.9
+constexpr int kDequantUnroll = BQ_DEQUANT_UNROLL;  // measured on C2 / C1 / C3: 1 -> 60.9 / 17.9 / 49.4 us, 2 -> 53.7 / 16.1 / 47.5, 4 -> 57.3 / 16.4 / 48.9
 
 template <int VPL, bool BF16>
 __global__ void __launch_bounds__(kThreads)

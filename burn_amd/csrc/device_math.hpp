@@ -27,6 +27,30 @@ __device__ __forceinline__ float scale_from_absmax(float amax, float span) {
   return (amax * 2.0f) / span;
 }
 
+// scale_to_dtype (crates/burn-std/src/tensor/quantization.rs:354-368): the smallest value the scale
+// dtype represents that is no smaller than s, as an f32. sdt: 0 f32 (identity), 1 f16, 2 bf16
+// (BQ_SCALE_*). NaN and the infinities pass through; a finite scale past the dtype's largest finite
+// value saturates to it.
+__device__ __forceinline__ float scale_round_up(float s, int sdt) {
+  if (sdt == 0) return s;
+  const uint32_t u = __float_as_uint(s), mag = u & 0x7FFFFFFFu;
+  if (mag >= 0x7F800000u) return s;
+  if (sdt == 2) {  // bf16: the upper 16 bits; rounding the magnitude up (s > 0) or truncating it (s < 0)
+    if ((u & 0xFFFFu) == 0u) return s;
+    if (u & 0x80000000u) return __uint_as_float(u & 0xFFFF0000u);
+    const uint32_t r = (u + 0xFFFFu) & 0xFFFF0000u;
+    return __uint_as_float(r >= 0x7F800000u ? 0x7F7F0000u : r);
+  }
+  // f16: 11 significant bits down to 2^-14, multiples of 2^-24 below; largest finite value 65504
+  int e = static_cast<int>(mag >> 23) - 127;
+  if (e < -14) e = -14;
+  if (e > 15) return s > 0.0f ? 65504.0f : -65504.0f;
+  const float q = __uint_as_float(static_cast<uint32_t>(e - 10 + 127) << 23);   // the spacing, a power of two
+  const float inv = __uint_as_float(static_cast<uint32_t>(10 - e + 127) << 23);
+  const float r = ceilf(s * inv) * q;  // both products exact
+  return r > 65504.0f ? 65504.0f : r;
+}
+
 // round half away from zero of a value already clamped to [-128, 128]. trunc(v + copysign(c, v))
 // with c = pred(0.5): adding 0.5 itself would carry pred(0.5) up to 1.0, every other case is
 // exact or rounds back below the next integer.

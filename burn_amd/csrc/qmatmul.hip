@@ -497,9 +497,10 @@ using namespace bq;
 
 static bool use_gemv(size_t m, int32_t lhs_dtype) { return m <= 16 && lhs_dtype == BQ_F32; }
 // Batch size from which the split-activation MFMA kernel beats the vector-ALU decode kernel on
-// the 4096 x 14336 weight. Q8S: about 23 us whatever M, against 21 us at M = 3, 23 at M = 4 and
-// 29 at M = 5. Q4S: about 21 us, against 17 us at M = 2 and about as much from M = 3.
-static size_t split_from_m(int value) { return value == BQ_Q8S ? 5 : 3; }
+// the 4096 x 14336 weight. Q8S: decode 16.5 / 18.7 / 20.3 / 22.6 us for M = 1..4, the matrix-core
+// kernel 21 us for M = 3 and 4 (its row-packed form, M <= 4) and 22-24.5 us above. Q4S: decode
+// 14.6 / 17.0 us for M = 1, 2, the matrix-core kernel 17.9 us for M = 3 and 4.
+static size_t split_from_m(int value) { return value == BQ_Q8S ? 4 : 3; }
 
 namespace bq {
 // Whether bqk_q_matmul has a fused kernel for this problem (else: dequantize + float matmul).

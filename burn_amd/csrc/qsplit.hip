@@ -75,11 +75,22 @@ template <int R>
 __device__ __forceinline__ float row_lane(uint32_t v) {
   return as_float(static_cast<uint32_t>(__builtin_amdgcn_update_dpp(0, static_cast<int>(v), 0x150 + R, 0xF, 0xF, false)));
 }
+// The value lane R of the caller's quad of 4 lanes holds (DPP quad_perm:[R,R,R,R]).
+template <int R>
+__device__ __forceinline__ float quad_lane(uint32_t v) {
+  return as_float(static_cast<uint32_t>(__builtin_amdgcn_update_dpp(0, static_cast<int>(v), R * 0x55, 0xF, 0xF, false)));
+}
 
 // MT: tiles of 16 activation rows (1 or 2): a lane prepares the split activations of rows c and
 // c + 16 and multiplies both against the same weight operands.
 // SB: log2 of (scale block / 32 columns): a scale serves 1, 2 or 4 of a wave's blocks of 32 columns.
-template <int VPL, bool PER_TENSOR, bool X_BF16, int MT, int SB = 0>
+// PK (M <= 4, one scale per 32 columns): the 16 rows of the A operand are 4 activation rows x the
+// wave's 4 blocks of 32 columns -- lane c prepares row c % 4 against the scales of block c / 4 -- so
+// the split activations are computed once per step instead of once per block (they are most of the
+// vector-ALU work: 32 of 60 instructions per 1024 weights). Every block's MFMAs then take the same
+// A operand, and of a block's accumulator only rows 4 u .. 4 u + 3 (the lanes with kg == u) are its
+// product; the others multiply another block's scales and are dropped.
+template <int VPL, bool PER_TENSOR, bool X_BF16, int MT, int SB = 0, bool PK = false>
 __global__ void __launch_bounds__(kSplitThreads)
 qsplit_kernel(const void* __restrict__ x, const uint32_t* __restrict__ w, const float* __restrict__ scales,
               size_t M, size_t K, size_t N, size_t k_per_wg, float* __restrict__ part) {
@@ -126,7 +137,10 @@ qsplit_kernel(const void* __restrict__ x, const uint32_t* __restrict__ w, const 
   const uint32_t w_row_bytes = static_cast<uint32_t>(NW * 4), s_row_bytes = static_cast<uint32_t>(spr * 4);
   const uint32_t w_lane = static_cast<uint32_t>(lane / LPR) * w_row_bytes + static_cast<uint32_t>(gc) * ROW_B +
                           static_cast<uint32_t>(lane % LPR) * 16u;
-  const uint32_t s_lane = static_cast<uint32_t>(8 * kg + (c & 7)) * s_row_bytes + static_cast<uint32_t>(gc * (4 >> SB)) * 4u;
+  static_assert(!PK || (MT == 1 && SB == 0 && !PER_TENSOR), "row packing: one tile of rows, one scale per 32 columns");
+  // PK: lane (row c % 4, block c / 4) loads that block's scale for k rows 8 kg + c % 4 and + 4
+  const uint32_t s_lane = PK ? static_cast<uint32_t>(8 * kg + (c & 3)) * s_row_bytes + static_cast<uint32_t>(gc * 4 + (c >> 2)) * 4u
+                             : static_cast<uint32_t>(8 * kg + (c & 7)) * s_row_bytes + static_cast<uint32_t>(gc * (4 >> SB)) * 4u;
   unsigned char* const slot = smem + slot_base + static_cast<uint32_t>(wave) * kSlotBytes;
   uint32_t slot_wr[NLOAD], slot_rd[kUnits];  // byte offsets in the slot: store i of a step; unit u, row 8 kg
 #pragma unroll
@@ -167,7 +181,10 @@ qsplit_kernel(const void* __restrict__ x, const uint32_t* __restrict__ w, const 
 #pragma unroll
     for (int i = 0; i < NLOAD; ++i)
       wl[buf][i] = __builtin_amdgcn_raw_buffer_load_b128(rsrc_w, wo, (row0 + static_cast<uint32_t>(RPI * i)) * w_row_bytes, 0);
-    if (!PER_TENSOR) {  // the 4, 2 or 1 scales of the group's row
+    if (PK) {
+      sq[buf] = vuint4{__builtin_amdgcn_raw_buffer_load_b32(rsrc_s, so, row0 * s_row_bytes, 0),
+                       __builtin_amdgcn_raw_buffer_load_b32(rsrc_s, so, (row0 + 4u) * s_row_bytes, 0), 0u, 0u};
+    } else if (!PER_TENSOR) {  // the 4, 2 or 1 scales of the group's row
       if (SB == 0) {
         sq[buf] = __builtin_amdgcn_raw_buffer_load_b128(rsrc_s, so, row0 * s_row_bytes, 0);
       } else if (SB == 1) {
@@ -191,7 +208,7 @@ qsplit_kernel(const void* __restrict__ x, const uint32_t* __restrict__ w, const 
     float xv[MT][8];
 #pragma unroll
     for (int t = 0; t < MT; ++t) {
-      const vfloat4* xp = reinterpret_cast<const vfloat4*>(xs + (c + 16 * t) * xpitch + kl);
+      const vfloat4* xp = reinterpret_cast<const vfloat4*>(xs + ((PK ? (c & 3) : c) + 16 * t) * xpitch + kl);
       const vfloat4 x0 = xp[0], x1 = xp[1];
       xv[t][0] = x0.x; xv[t][1] = x0.y; xv[t][2] = x0.z; xv[t][3] = x0.w;
       xv[t][4] = x1.x; xv[t][5] = x1.y; xv[t][6] = x1.z; xv[t][7] = x1.w;
@@ -205,6 +222,15 @@ qsplit_kernel(const void* __restrict__ x, const uint32_t* __restrict__ w, const 
 #pragma unroll
       for (int r = 0; r < 8; ++r) wq[u][r] = *reinterpret_cast<const uint32_t*>(slot + slot_rd[u] + ROW_B * r);
     uint32_t hi[MT][4], lo[MT][4];
+    if (PK) {
+      const uint32_t a = sq[buf].x, b = sq[buf].y;
+      const float sr[8] = {quad_lane<0>(a), quad_lane<1>(a), quad_lane<2>(a), quad_lane<3>(a),
+                           quad_lane<0>(b), quad_lane<1>(b), quad_lane<2>(b), quad_lane<3>(b)};
+      float v[8];
+#pragma unroll
+      for (int r = 0; r < 8; ++r) v[r] = xv[0][r] * sr[r];
+      split(v, hi[0], lo[0]);
+    }
     if (PER_TENSOR) {
 #pragma unroll
       for (int t = 0; t < MT; ++t) {
@@ -216,7 +242,7 @@ qsplit_kernel(const void* __restrict__ x, const uint32_t* __restrict__ w, const 
     }
 #pragma unroll
     for (int u = 0; u < kUnits; ++u) {
-      if (!PER_TENSOR) {
+      if (!PER_TENSOR && !PK) {
         const uint32_t sv = sq[buf][u >> SB];
         const float sr[8] = {row_lane<0>(sv), row_lane<1>(sv), row_lane<2>(sv), row_lane<3>(sv),
                              row_lane<4>(sv), row_lane<5>(sv), row_lane<6>(sv), row_lane<7>(sv)};
@@ -326,6 +352,9 @@ qsplit_kernel(const void* __restrict__ x, const uint32_t* __restrict__ w, const 
   constexpr uint32_t SP = kTileCols + 4;  // pitch in floats
   const uint32_t cell0 = static_cast<uint32_t>(4 * kg) * SP + static_cast<uint32_t>(g) * kGroupCols +
                          static_cast<uint32_t>(VPL * (c % WPB) + c / WPB);
+  // PK: block u's product sits in rows 4 u .. 4 u + 3 of its accumulators, i.e. in the lanes with
+  // kg == u, element i = activation row i.
+  const uint32_t cellp = static_cast<uint32_t>(g) * kGroupCols + static_cast<uint32_t>(VPL * (c % WPB) + c / WPB);
   if (h == 1) {
 #pragma unroll
     for (int t = 0; t < MT; ++t)
@@ -334,7 +363,13 @@ qsplit_kernel(const void* __restrict__ x, const uint32_t* __restrict__ w, const 
 #pragma unroll
         for (int p = 0; p < 2; ++p)
 #pragma unroll
-          for (int i = 0; i < 4; ++i) stage[cell0 + (16 * t + i) * SP + 32 * u + (VPL / 2) * p] = acc[t][u][p][i];
+          for (int i = 0; i < 4; ++i) {
+            if (PK) {
+              if (kg == u) stage[cellp + i * SP + 32 * u + (VPL / 2) * p] = acc[t][u][p][i];
+            } else {
+              stage[cell0 + (16 * t + i) * SP + 32 * u + (VPL / 2) * p] = acc[t][u][p][i];
+            }
+          }
   }
   __syncthreads();
   if (h == 0) {
@@ -345,7 +380,13 @@ qsplit_kernel(const void* __restrict__ x, const uint32_t* __restrict__ w, const 
 #pragma unroll
         for (int p = 0; p < 2; ++p)
 #pragma unroll
-          for (int i = 0; i < 4; ++i) stage[cell0 + (16 * t + i) * SP + 32 * u + (VPL / 2) * p] += acc[t][u][p][i];
+          for (int i = 0; i < 4; ++i) {
+            if (PK) {
+              if (kg == u) stage[cellp + i * SP + 32 * u + (VPL / 2) * p] += acc[t][u][p][i];
+            } else {
+              stage[cell0 + (16 * t + i) * SP + 32 * u + (VPL / 2) * p] += acc[t][u][p][i];
+            }
+          }
   }
   __syncthreads();
   {
@@ -402,17 +443,18 @@ bq_status launch_qsplit(const void* x, int x_dtype, const uint32_t* w, const flo
   const size_t mt = m > 16 ? 2 : 1;
   const size_t lds = 16 * mt * (kMaxSlice + 4) * sizeof(float) + kSplitWaves * kSlotBytes;
   dim3 grid(p.tiles, p.slices), tb(kSplitThreads);
-#define BQ_SPLIT2(V, PT, XB, T, S)                                                                          \
+#define BQ_SPLIT3(V, PT, XB, T, S, P)                                                              \
   do {                                                                                            \
-    auto kernel = qsplit_kernel<V, PT, XB, T, S>;                                                           \
+    auto kernel = qsplit_kernel<V, PT, XB, T, S, P>;                                              \
     /* more than the default 64 KiB: checked against what the device grants, else refused here */ \
     BQ_TRY(configure_dynamic_lds(reinterpret_cast<const void*>(kernel), lds, "qsplit_kernel"));   \
     hipLaunchKernelGGL(kernel, grid, tb, lds, st, x, w, scales, m, k, n, p.k_per_wg, part);       \
   } while (0)
 #define BQ_SPLIT(V, PT, XB, S)                  \
-  if (mt == 2) BQ_SPLIT2(V, PT, XB, 2, S); else BQ_SPLIT2(V, PT, XB, 1, S)
+  if (mt == 2) BQ_SPLIT3(V, PT, XB, 2, S, false); else BQ_SPLIT3(V, PT, XB, 1, S, false)
 #define BQ_SPLIT_B(V, XB)                                \
   if (per_tensor) BQ_SPLIT(V, true, XB, 0);              \
+  else if (block == 32 && m <= 4) BQ_SPLIT3(V, false, XB, 1, 0, true); /* row packing */ \
   else if (block == 32) BQ_SPLIT(V, false, XB, 0);       \
   else if (block == 64) BQ_SPLIT(V, false, XB, 1);       \
   else BQ_SPLIT(V, false, XB, 2)
@@ -421,7 +463,7 @@ bq_status launch_qsplit(const void* x, int x_dtype, const uint32_t* w, const flo
   if (value == BQ_Q8S) { BQ_SPLIT_V(4) } else { BQ_SPLIT_V(8) }
 #undef BQ_SPLIT_V
 #undef BQ_SPLIT_B
-#undef BQ_SPLIT2
+#undef BQ_SPLIT3
 #undef BQ_SPLIT
   BQ_HIP(hipGetLastError());
   *slices_out = p.slices;

@@ -16,7 +16,29 @@ namespace bq {
 
 namespace {
 
-constexpr int kThreads = 256;
+// Tunables (the defaults are the measured best; overridable at compile time for sweeps).
+#ifndef BQ_QUANT_THREADS
+#define BQ_QUANT_THREADS 256
+#endif
+#ifndef BQ_BLOCK_THREADS
+#define BQ_BLOCK_THREADS 64
+#endif
+#ifndef BQ_BLOCK_UNROLL
+#define BQ_BLOCK_UNROLL 4
+#endif
+#ifndef BQ_TENSOR_UNROLL
+#define BQ_TENSOR_UNROLL 4
+#endif
+#ifndef BQ_ABSMAX_UNROLL
+#define BQ_ABSMAX_UNROLL 8
+#endif
+#ifndef BQ_ABSMAX_NT
+#define BQ_ABSMAX_NT 0
+#endif
+#ifndef BQ_QUANT_NT_STORE
+#define BQ_QUANT_NT_STORE 1
+#endif
+constexpr int kThreads = BQ_QUANT_THREADS;
 
 template <int VPL>
 struct Vals {
@@ -82,27 +104,32 @@ __device__ __forceinline__ uint32_t quantize_pack(const Vals<VPL>& a, float s_st
 }
 
 // ---- run-block schemes: B = LANES * VPL consecutive elements per scale ------------------------
-// A workgroup owns a contiguous chunk of kThreads * U words; lane t takes words t, t + 256, ...
+// A workgroup of T threads owns a contiguous chunk of T * U words; lane t takes words t, t + T, ...
 // of the chunk, so every load/store instruction of a wave is one contiguous 1 KiB / 256 B run and
-// U independent 128-bit loads are in flight per lane before any arithmetic starts. Measured on
-// the [8192, 8192] tensor: U = 1 61.4 us, U = 2 57.9 us, U = 4 59.0 us, U = 8 61.3 us. A fixed grid
-// of 1024-4096 workgroups that walk the chunks with a stride and load the next chunk ahead of
-// the arithmetic is slower (63-67 us): many short workgroups keep more loads in flight.
-constexpr int kBlockUnroll = 2;        // run-block kernel
-constexpr int kTensorUnroll = 4;       // per-tensor second pass
+// U independent 128-bit loads are in flight per lane before any arithmetic starts. The packed
+// words leave with non-temporal stores (like the loads: nothing here is read again by this
+// kernel); with plain stores the same shapes are 5 % slower. Measured on the [8192, 8192] tensor
+// (one box, graph replays, non-temporal stores), T x U: 64 x 1 73.2 us, 64 x 2 55.4, 64 x 4 55.1,
+// 64 x 8 57.9, 128 x 2 57.5, 128 x 4 55.7, 128 x 8 57.9, 256 x 2 57.1, 256 x 4 56.2; with plain
+// stores 256 x 2 took 60.0 us. A fixed grid of 1024-4096 workgroups that walk the chunks with a
+// stride and load the next chunk ahead of the arithmetic is slower (63-67 us): many short
+// workgroups keep more loads in flight.
+constexpr int kBlockThreads = BQ_BLOCK_THREADS;      // run-block kernel
+constexpr int kBlockUnroll = BQ_BLOCK_UNROLL;
+constexpr int kTensorUnroll = BQ_TENSOR_UNROLL;      // per-tensor second pass
 
 template <int VPL, int LANES, bool DYNAMIC>
-__global__ void __launch_bounds__(kThreads)
+__global__ void __launch_bounds__(kBlockThreads)
 quantize_block_kernel(const float* __restrict__ x, size_t words, uint32_t* __restrict__ out,
-                      float* __restrict__ scales_out, const float* __restrict__ scales_in) {
+                      float* __restrict__ scales_out, const float* __restrict__ scales_in, int sdt) {
   constexpr int U = kBlockUnroll;
   constexpr int QMAX = (VPL == 4) ? 127 : 7;
   constexpr float SPAN = 2.0f * QMAX;
-  const size_t base = static_cast<size_t>(blockIdx.x) * (kThreads * U) + threadIdx.x;
+  const size_t base = static_cast<size_t>(blockIdx.x) * (kBlockThreads * U) + threadIdx.x;
   Vals<VPL> a[U];
 #pragma unroll
   for (int u = 0; u < U; ++u) {
-    const size_t w = base + static_cast<size_t>(u) * kThreads;
+    const size_t w = base + static_cast<size_t>(u) * kBlockThreads;
     if (w < words) {
       a[u] = load_vals<VPL>(x, w);
     } else {
@@ -114,12 +141,15 @@ quantize_block_kernel(const float* __restrict__ x, size_t words, uint32_t* __res
   // in range (or out of range) together; the cross-lane max runs in every lane either way.
 #pragma unroll
   for (int u = 0; u < U; ++u) {
-    const size_t w = base + static_cast<size_t>(u) * kThreads;
+    const size_t w = base + static_cast<size_t>(u) * kBlockThreads;
     uint32_t word;
     float s;
     if (DYNAMIC) {
       const float m = group_max<LANES>(absmax_vals<VPL>(a[u]));
-      if (absmax_fast_ok(m)) {
+      if (sdt != BQ_SCALE_F32) {  // f16 / bf16 scales: divide by the scale as it will be stored
+        s = scale_round_up(absmax_fast_ok(m) ? scale_from_absmax_fast<QMAX>(m) : scale_from_absmax(m, SPAN), sdt);
+        word = quantize_pack<VPL>(a[u], s);
+      } else if (absmax_fast_ok(m)) {
         s = scale_from_absmax_fast<QMAX>(m);
         word = quantize_pack_recip<VPL, false>(a[u], s, recip_exact(s));
       } else {
@@ -132,7 +162,7 @@ quantize_block_kernel(const float* __restrict__ x, size_t words, uint32_t* __res
     }
     if (w < words) {
       if (DYNAMIC && (w & (LANES - 1)) == 0) scales_out[w / LANES] = s;
-      out[w] = word;
+      if (BQ_QUANT_NT_STORE) __builtin_nontemporal_store(word, out + w); else out[w] = word;
     }
   }
 }
@@ -142,7 +172,7 @@ quantize_block_kernel(const float* __restrict__ x, size_t words, uint32_t* __res
 // a grid stride (plain loads: the second pass re-reads the tensor, so it is left in the caches;
 // the next chunk's loads are issued before the current one is reduced) and stores max|x| of what
 // it saw to its own cell. No atomics, so the cells need no initialisation.
-constexpr int kAbsmaxUnroll = 8;
+constexpr int kAbsmaxUnroll = BQ_ABSMAX_UNROLL;
 
 // max over the workgroup, in every thread (one call per kernel: the LDS cells are not reused)
 __device__ __forceinline__ float workgroup_max(float m) {
@@ -167,7 +197,7 @@ absmax_kernel(const float* __restrict__ x, size_t n, uint32_t* __restrict__ absm
 #pragma unroll
     for (int u = 0; u < U; ++u) {
       const size_t i = base + static_cast<size_t>(u) * kThreads;
-      t[u] = (i < n4) ? p[i] : vfloat4{0.f, 0.f, 0.f, 0.f};
+      t[u] = (i < n4) ? (BQ_ABSMAX_NT ? __builtin_nontemporal_load(p + i) : p[i]) : vfloat4{0.f, 0.f, 0.f, 0.f};
     }
   };
   float m = 0.0f;
@@ -191,10 +221,9 @@ absmax_kernel(const float* __restrict__ x, size_t n, uint32_t* __restrict__ absm
 
 // max over the BQ_ABSMAX_CELLS cells, in every thread of a workgroup of kThreads threads.
 __device__ __forceinline__ float absmax_from_cells(const uint32_t* __restrict__ cells) {
-  static_assert(BQ_ABSMAX_CELLS % kThreads == 0, "whole cells per thread");
   float m = 0.0f;
 #pragma unroll
-  for (int i = 0; i < BQ_ABSMAX_CELLS / kThreads; ++i) m = fmaxf(m, __uint_as_float(cells[threadIdx.x + i * kThreads]));
+  for (int i = static_cast<int>(threadIdx.x); i < BQ_ABSMAX_CELLS; i += kThreads) m = fmaxf(m, __uint_as_float(cells[i]));
   return workgroup_max(m);
 }
 
@@ -210,8 +239,8 @@ absmax_scalar_kernel(const float* __restrict__ x, size_t n, uint32_t* __restrict
 }
 
 __global__ void __launch_bounds__(kThreads)
-scale_from_cells_kernel(const uint32_t* __restrict__ cells, float span, float* __restrict__ scale_out) {
-  const float s = scale_from_absmax(absmax_from_cells(cells), span);
+scale_from_cells_kernel(const uint32_t* __restrict__ cells, float span, int sdt, float* __restrict__ scale_out) {
+  const float s = scale_round_up(scale_from_absmax(absmax_from_cells(cells), span), sdt);
   if (threadIdx.x == 0) scale_out[0] = s;
 }
 
@@ -228,7 +257,7 @@ __global__ void scales_from_absmax_kernel(const float* __restrict__ amax, size_t
 template <int VPL, bool FROM_ABSMAX>
 __global__ void __launch_bounds__(kThreads)
 quantize_tensor_kernel(const float* __restrict__ x, size_t n, const float* __restrict__ scale,
-                       float* __restrict__ scale_out, uint32_t* __restrict__ out) {
+                       float* __restrict__ scale_out, uint32_t* __restrict__ out, int sdt) {
   constexpr int U = kTensorUnroll;
   constexpr float SPAN = (VPL == 4) ? 254.0f : 14.0f;
   constexpr float QMAX = (VPL == 4) ? 127.0f : 7.0f;
@@ -246,7 +275,7 @@ quantize_tensor_kernel(const float* __restrict__ x, size_t n, const float* __res
     }
   }
   const float s_stored =
-      FROM_ABSMAX ? scale_from_absmax(absmax_from_cells(reinterpret_cast<const uint32_t*>(scale)), SPAN)
+      FROM_ABSMAX ? scale_round_up(scale_from_absmax(absmax_from_cells(reinterpret_cast<const uint32_t*>(scale)), SPAN), sdt)
                   : scale[0];
   if (FROM_ABSMAX && blockIdx.x == 0 && threadIdx.x == 0) scale_out[0] = s_stored;
   const float s = valid_scale(s_stored);
@@ -256,7 +285,10 @@ quantize_tensor_kernel(const float* __restrict__ x, size_t n, const float* __res
   for (int u = 0; u < U; ++u) {
     const size_t w = base + static_cast<size_t>(u) * kThreads;
     if (w < words)
-      out[w] = fast ? quantize_pack_recip<VPL, true>(a[u], s, r) : quantize_pack_div<VPL>(a[u], s);
+    {
+      const uint32_t word = fast ? quantize_pack_recip<VPL, true>(a[u], s, r) : quantize_pack_div<VPL>(a[u], s);
+      if (BQ_QUANT_NT_STORE) __builtin_nontemporal_store(word, out + w); else out[w] = word;
+    }
   }
   // native i8 store with n % 4 != 0: the last 1..3 values, one byte each
   if (VPL == 4 && blockIdx.x == 0 && threadIdx.x == 0) {
@@ -297,7 +329,7 @@ __device__ __forceinline__ size_t rect_block_of(const RectDims& d, size_t index)
 
 // One thread per block: max |x| over the block rectangle -> scale.
 __global__ void rect_scales_kernel(const float* __restrict__ x, RectDims d, size_t nblocks,
-                                   size_t block_elems, float span, float* __restrict__ scales) {
+                                   size_t block_elems, float span, int sdt, float* __restrict__ scales) {
   size_t b = static_cast<size_t>(blockIdx.x) * blockDim.x + threadIdx.x;
   if (b >= nblocks) return;
   // origin of block b
@@ -318,7 +350,7 @@ __global__ void rect_scales_kernel(const float* __restrict__ x, RectDims d, size
     }
     m = fmaxf(m, fabsf(x[idx]));
   }
-  scales[b] = scale_from_absmax(m, span);
+  scales[b] = scale_round_up(scale_from_absmax(m, span), sdt);
 }
 
 // One thread per output word; every value looks its own block up, so words may straddle blocks.
@@ -356,14 +388,14 @@ inline unsigned grid_for(size_t items, unsigned cap) {
 
 template <int VPL, bool DYNAMIC>
 bq_status launch_block(const float* x, size_t n, int block, uint32_t* out, float* scales_out,
-                       const float* scales_in, hipStream_t st) {
+                       const float* scales_in, int sdt, hipStream_t st) {
   const size_t words = n / VPL;
   const int lanes = block / VPL;
-  const unsigned grid = static_cast<unsigned>((words + kThreads * kBlockUnroll - 1) / (kThreads * kBlockUnroll));
+  const unsigned grid = static_cast<unsigned>((words + kBlockThreads * kBlockUnroll - 1) / (kBlockThreads * kBlockUnroll));
 #define BQ_CASE(L)                                                                         \
   case L:                                                                                  \
-    hipLaunchKernelGGL((quantize_block_kernel<VPL, L, DYNAMIC>), dim3(grid), dim3(kThreads), \
-                       0, st, x, words, out, scales_out, scales_in);                       \
+    hipLaunchKernelGGL((quantize_block_kernel<VPL, L, DYNAMIC>), dim3(grid), dim3(kBlockThreads), \
+                       0, st, x, words, out, scales_out, scales_in, sdt);                  \
     break;
   switch (lanes) {
     BQ_CASE(1) BQ_CASE(2) BQ_CASE(4) BQ_CASE(8) BQ_CASE(16) BQ_CASE(32) BQ_CASE(64)
@@ -445,7 +477,7 @@ __global__ void __launch_bounds__(256) copy16_kernel(const vuint4* __restrict__ 
 }
 
 bq_status launch_quantize_rect(const float* x, const size_t* shape, int rank, const size_t* blk,
-                               int value, int store, bool dynamic, void* values, float* scales,
+                               int value, int store, bool dynamic, int sdt, void* values, float* scales,
                                hipStream_t st) {
   RectDims d{};
   d.rank = blk ? rank : 0;
@@ -464,7 +496,7 @@ bq_status launch_quantize_rect(const float* x, const size_t* shape, int rank, co
     RectDims dd = d;
     dd.rank = rank;  // per-tensor: one block spanning everything
     hipLaunchKernelGGL(rect_scales_kernel, dim3((nblocks + 63) / 64), dim3(64), 0, st, x, dd,
-                       nblocks, block_elems, span, scales);
+                       nblocks, block_elems, span, sdt, scales);
     BQ_HIP(hipGetLastError());
   }
   const size_t last = rank ? shape[rank - 1] : 1;
@@ -479,6 +511,73 @@ bq_status launch_quantize_rect(const float* x, const size_t* shape, int rank, co
   else
     hipLaunchKernelGGL(rect_quantize_kernel<4>, grid, tb, 0, st, x, d, last, wpl, total, native,
                        scales, static_cast<uint32_t*>(values));
+  BQ_HIP(hipGetLastError());
+  return BQ_OK;
+}
+
+// ---- scales in a 2-byte dtype ------------------------------------------------------------------
+// Tensors keep their scales as f32 on the device, holding values the scale dtype represents exactly
+// (rounded up at quantize time, or widened when a blob is loaded); the 2-byte form only exists on
+// the wire.
+__global__ void round_scales_kernel(const float* __restrict__ src, float* __restrict__ dst, size_t n, int sdt) {
+  const size_t i = static_cast<size_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+  if (i < n) dst[i] = scale_round_up(src[i], sdt);
+}
+
+// f32 -> f16 bits of a value f16 represents exactly (or an infinity / NaN)
+__device__ __forceinline__ uint16_t f16_bits_exact(float v) {
+  const uint32_t u = __float_as_uint(v), sign = (u >> 16) & 0x8000u, mag = u & 0x7FFFFFFFu;
+  if (mag >= 0x7F800000u) return static_cast<uint16_t>(sign | 0x7C00u | (mag > 0x7F800000u ? 0x200u : 0u));
+  if (mag < 0x38800000u) {  // below 2^-14: a multiple of 2^-24
+    const float t = fabsf(v) * 16777216.0f;
+    return static_cast<uint16_t>(sign | static_cast<uint32_t>(t));
+  }
+  return static_cast<uint16_t>(sign | ((mag - 0x38000000u) >> 13));
+}
+
+__device__ __forceinline__ float f16_bits_to_f32(uint16_t h) {
+  const uint32_t sign = (static_cast<uint32_t>(h) & 0x8000u) << 16, ex = (h >> 10) & 0x1Fu, man = h & 0x3FFu;
+  if (ex == 0) {
+    const float t = static_cast<float>(man) * 5.9604644775390625e-8f;  // man * 2^-24, exact
+    return __uint_as_float(sign | __float_as_uint(t));
+  }
+  if (ex == 31) return __uint_as_float(sign | 0x7F800000u | (man << 13));
+  return __uint_as_float(sign | ((ex + 112u) << 23) | (man << 13));
+}
+
+__global__ void scales_to_wire_kernel(const float* __restrict__ src, uint16_t* __restrict__ dst, size_t n, int sdt) {
+  const size_t i = static_cast<size_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+  if (i >= n) return;
+  // (a scale that did not pass through scale_round_up, e.g. given by hand: rounded up here as well)
+  const float v = scale_round_up(src[i], sdt);
+  dst[i] = sdt == 2 ? static_cast<uint16_t>(__float_as_uint(v) >> 16) : f16_bits_exact(v);
+}
+
+__global__ void scales_from_wire_kernel(const uint16_t* __restrict__ src, float* __restrict__ dst, size_t n, int sdt) {
+  const size_t i = static_cast<size_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+  if (i >= n) return;
+  dst[i] = sdt == 2 ? __uint_as_float(static_cast<uint32_t>(src[i]) << 16) : f16_bits_to_f32(src[i]);
+}
+
+bq_status launch_round_scales(const float* src, float* dst, size_t n, int sdt, hipStream_t st) {
+  if (n == 0) return BQ_OK;
+  hipLaunchKernelGGL(round_scales_kernel, dim3(static_cast<unsigned>((n + 255) / 256)), dim3(256), 0, st, src, dst, n, sdt);
+  BQ_HIP(hipGetLastError());
+  return BQ_OK;
+}
+
+bq_status launch_scales_to_wire(const float* src, void* dst, size_t n, int sdt, hipStream_t st) {
+  if (n == 0) return BQ_OK;
+  hipLaunchKernelGGL(scales_to_wire_kernel, dim3(static_cast<unsigned>((n + 255) / 256)), dim3(256), 0, st, src,
+                     static_cast<uint16_t*>(dst), n, sdt);
+  BQ_HIP(hipGetLastError());
+  return BQ_OK;
+}
+
+bq_status launch_scales_from_wire(const void* src, float* dst, size_t n, int sdt, hipStream_t st) {
+  if (n == 0) return BQ_OK;
+  hipLaunchKernelGGL(scales_from_wire_kernel, dim3(static_cast<unsigned>((n + 255) / 256)), dim3(256), 0, st,
+                     static_cast<const uint16_t*>(src), dst, n, sdt);
   BQ_HIP(hipGetLastError());
   return BQ_OK;
 }
@@ -593,7 +692,7 @@ static bq_status check_value_store(int32_t value, int32_t store, size_t n) {
 // the derived scale (saves the separate scales_from_absmax launch in quantize_dynamic).
 static bq_status quantize_per_tensor_impl(const float* x, size_t n, const float* scale,
                                           bool from_absmax, float* scale_out, int32_t value,
-                                          int32_t store, void* values, hipStream_t st) {
+                                          int32_t store, void* values, int sdt, hipStream_t st) {
   BQ_TRY(check_value_store(value, store, n));
   if (n == 0) return BQ_OK;
   if (!aligned16(x) || (reinterpret_cast<uintptr_t>(values) & 3u)) {
@@ -601,7 +700,7 @@ static bq_status quantize_per_tensor_impl(const float* x, size_t n, const float*
       BQ_FAIL(BQ_ERR_SHAPE, "Q4S quantize needs a 16-byte aligned input and 4-byte aligned output");
     if (from_absmax) {
       hipLaunchKernelGGL(scale_from_cells_kernel, dim3(1), dim3(kThreads), 0, st,
-                         reinterpret_cast<const uint32_t*>(scale), 254.0f, scale_out);
+                         reinterpret_cast<const uint32_t*>(scale), 254.0f, sdt, scale_out);
       scale = scale_out;
     }
     hipLaunchKernelGGL(quantize_tensor_scalar_kernel, dim3(grid_for(n, 65536u)), dim3(kThreads), 0, st, x,
@@ -617,14 +716,14 @@ static bq_status quantize_per_tensor_impl(const float* x, size_t n, const float*
   uint32_t* out = static_cast<uint32_t*>(values);
   if (value == BQ_Q8S) {
     if (from_absmax)
-      hipLaunchKernelGGL((quantize_tensor_kernel<4, true>), grid, tb, 0, st, x, n, scale, scale_out, out);
+      hipLaunchKernelGGL((quantize_tensor_kernel<4, true>), grid, tb, 0, st, x, n, scale, scale_out, out, sdt);
     else
-      hipLaunchKernelGGL((quantize_tensor_kernel<4, false>), grid, tb, 0, st, x, n, scale, scale_out, out);
+      hipLaunchKernelGGL((quantize_tensor_kernel<4, false>), grid, tb, 0, st, x, n, scale, scale_out, out, sdt);
   } else {
     if (from_absmax)
-      hipLaunchKernelGGL((quantize_tensor_kernel<8, true>), grid, tb, 0, st, x, n, scale, scale_out, out);
+      hipLaunchKernelGGL((quantize_tensor_kernel<8, true>), grid, tb, 0, st, x, n, scale, scale_out, out, sdt);
     else
-      hipLaunchKernelGGL((quantize_tensor_kernel<8, false>), grid, tb, 0, st, x, n, scale, scale_out, out);
+      hipLaunchKernelGGL((quantize_tensor_kernel<8, false>), grid, tb, 0, st, x, n, scale, scale_out, out, sdt);
   }
   BQ_HIP(hipGetLastError());
   return BQ_OK;
@@ -639,7 +738,7 @@ extern "C" bq_status bqk_quantize_per_tensor_from_absmax(const float* x, size_t 
   BQ_NOTNULL(scale_out);
   BQ_NOTNULL(values);
   return quantize_per_tensor_impl(x, n, reinterpret_cast<const float*>(absmax_cells), true, scale_out,
-                                  value, store, values, static_cast<hipStream_t>(stream));
+                                  value, store, values, BQ_SCALE_F32, static_cast<hipStream_t>(stream));
 }
 
 extern "C" bq_status bqk_quantize_per_tensor(const float* x, size_t n, const float* scale,
@@ -648,7 +747,7 @@ extern "C" bq_status bqk_quantize_per_tensor(const float* x, size_t n, const flo
   BQ_NOTNULL(x);
   BQ_NOTNULL(scale);
   BQ_NOTNULL(values);
-  return quantize_per_tensor_impl(x, n, scale, false, nullptr, value, store, values,
+  return quantize_per_tensor_impl(x, n, scale, false, nullptr, value, store, values, BQ_SCALE_F32,
                                   static_cast<hipStream_t>(stream));
 }
 
@@ -676,8 +775,8 @@ extern "C" bq_status bqk_quantize_dynamic_block(const float* x, size_t n, int32_
   if (n == 0) return BQ_OK;
   hipStream_t st = static_cast<hipStream_t>(stream);
   if (value == BQ_Q8S)
-    return launch_block<4, true>(x, n, block, static_cast<uint32_t*>(values), scales, nullptr, st);
-  return launch_block<8, true>(x, n, block, static_cast<uint32_t*>(values), scales, nullptr, st);
+    return launch_block<4, true>(x, n, block, static_cast<uint32_t*>(values), scales, nullptr, BQ_SCALE_F32, st);
+  return launch_block<8, true>(x, n, block, static_cast<uint32_t*>(values), scales, nullptr, BQ_SCALE_F32, st);
 }
 
 extern "C" bq_status bqk_quantize_block(const float* x, size_t n, int32_t block,
@@ -690,8 +789,8 @@ extern "C" bq_status bqk_quantize_block(const float* x, size_t n, int32_t block,
   if (n == 0) return BQ_OK;
   hipStream_t st = static_cast<hipStream_t>(stream);
   if (value == BQ_Q8S)
-    return launch_block<4, false>(x, n, block, static_cast<uint32_t*>(values), nullptr, scales, st);
-  return launch_block<8, false>(x, n, block, static_cast<uint32_t*>(values), nullptr, scales, st);
+    return launch_block<4, false>(x, n, block, static_cast<uint32_t*>(values), nullptr, scales, BQ_SCALE_F32, st);
+  return launch_block<8, false>(x, n, block, static_cast<uint32_t*>(values), nullptr, scales, BQ_SCALE_F32, st);
 }
 
 
@@ -708,3 +807,25 @@ extern "C" bq_status bqk_copy(const void* src, void* dst, size_t bytes, void* st
   BQ_HIP(hipGetLastError());
   return BQ_OK;
 }
+
+namespace bq {
+
+// The handle level's entry into the fused kernels, with the scheme's scale dtype.
+bq_status launch_quantize_per_tensor(const float* x, size_t n, const float* scale_or_cells, bool from_absmax,
+                                     float* scale_out, int value, int store, void* values, int sdt, hipStream_t st) {
+  return quantize_per_tensor_impl(x, n, scale_or_cells, from_absmax, scale_out, value, store, values, sdt, st);
+}
+
+bq_status launch_quantize_run_block(const float* x, size_t n, int block, const float* scales_in, float* scales_out,
+                                    int value, int store, void* values, int sdt, hipStream_t st) {
+  BQ_TRY(check_block_args(x, n, block, value, store, values));
+  if (n == 0) return BQ_OK;
+  uint32_t* out = static_cast<uint32_t*>(values);
+  if (scales_in == nullptr)
+    return value == BQ_Q8S ? launch_block<4, true>(x, n, block, out, scales_out, nullptr, sdt, st)
+                           : launch_block<8, true>(x, n, block, out, scales_out, nullptr, sdt, st);
+  return value == BQ_Q8S ? launch_block<4, false>(x, n, block, out, nullptr, scales_in, sdt, st)
+                         : launch_block<8, false>(x, n, block, out, nullptr, scales_in, sdt, st);
+}
+
+}  // namespace bq

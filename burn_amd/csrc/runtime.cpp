@@ -58,6 +58,9 @@ static size_t value_bytes(const bq_scheme& s, const size_t* shape, int rank) {
   return 4 * lines * ((shape[rank - 1] + nq - 1) / nq);
 }
 
+// scale_size (crates/burn-std/src/tensor/quantization.rs:409-416): bytes per stored scale on the wire.
+static size_t scale_size(const bq_scheme& s) { return s.scale_dtype == BQ_SCALE_F32 ? 4 : 2; }
+
 // What the backend accepts: the same conditions under which the reference backends panic.
 // `storable`: also require what a packed device tensor needs (whole words along the last dim). The
 // length formula alone (quantized_data_len) pads a ragged last dim to whole words instead.
@@ -65,8 +68,8 @@ static bq_status check_scheme(const bq_scheme& s, const size_t* shape, int rank,
   if (rank < 1 || rank > BQ_MAX_RANK) BQ_FAIL(BQ_ERR_SHAPE, "rank %d outside 1..%d", rank, BQ_MAX_RANK);
   if (!value_known(s.value))
     BQ_FAIL(BQ_ERR_UNSUPPORTED_SCHEME, "Quantization not supported for value %d (Q8S and Q4S are)", s.value);
-  if (s.scale_dtype != BQ_SCALE_F32)
-    BQ_FAIL(BQ_ERR_UNSUPPORTED_SCHEME, "only f32 scales are supported");
+  if (s.scale_dtype != BQ_SCALE_F32 && s.scale_dtype != BQ_SCALE_F16 && s.scale_dtype != BQ_SCALE_BF16)
+    BQ_FAIL(BQ_ERR_UNSUPPORTED_SCHEME, "scale dtype %d is not supported (f32, f16 and bf16 are)", s.scale_dtype);
   if (s.level != BQ_LEVEL_TENSOR && s.level != BQ_LEVEL_BLOCK)
     BQ_FAIL(BQ_ERR_UNSUPPORTED_SCHEME, "unknown quantization level %d", s.level);
   if (s.store == BQ_STORE_NATIVE) {
@@ -561,7 +564,7 @@ extern "C" bq_status bq_quantized_data_len(const bq_scheme* scheme, const size_t
   // (a zero block extent, a dim the block does not divide, an unknown store or level are refused
   // here; a ragged last dim is not: the formula pads it to whole words, burn-store's data_len cases)
   BQ_TRY(check_scheme(*scheme, shape, rank, false));
-  *len_out = value_bytes(*scheme, shape, rank) + 4 * num_params(*scheme, shape, rank);
+  *len_out = value_bytes(*scheme, shape, rank) + scale_size(*scheme) * num_params(*scheme, shape, rank);
   return BQ_OK;
 }
 
@@ -574,7 +577,8 @@ extern "C" bq_status bq_q_from_data(bq_device* dev, const uint8_t* bytes, size_t
   BQ_NOTNULL(out);
   bq_tensor* t = nullptr;
   BQ_TRY(new_quantized(dev, *scheme, shape, rank, &t));
-  const size_t need = t->value_bytes + 4 * t->num_scales;
+  const size_t ssz = scale_size(*scheme);
+  const size_t need = t->value_bytes + ssz * t->num_scales;
   if (len != need) {
     bq_tensor_release(t);
     BQ_FAIL(BQ_ERR_SIZE, "quantized tensor data is %zu bytes, its scheme and shape need %zu", len, need);
@@ -585,13 +589,25 @@ extern "C" bq_status bq_q_from_data(bq_device* dev, const uint8_t* bytes, size_t
   }
   hipError_t e = hipSuccess;
   if (t->value_bytes) e = hipMemcpyAsync(t->data, bytes, t->value_bytes, hipMemcpyHostToDevice, dev->stream);
-  if (e == hipSuccess)
-    e = hipMemcpyAsync(t->scales(), bytes + t->value_bytes, 4 * t->num_scales, hipMemcpyHostToDevice,
-                       dev->stream);
+  bq_status rc = BQ_OK;
+  if (e == hipSuccess && ssz == 4) {
+    e = hipMemcpyAsync(t->scales(), bytes + t->value_bytes, 4 * t->num_scales, hipMemcpyHostToDevice, dev->stream);
+  } else if (e == hipSuccess) {
+    // 2-byte scales: staged in a device block, widened (exactly) to the f32 the kernels read
+    void* stage = nullptr;
+    size_t stage_bytes = 0;
+    rc = dev->alloc(2 * t->num_scales, &stage, &stage_bytes);
+    if (rc == BQ_OK) {
+      e = hipMemcpyAsync(stage, bytes + t->value_bytes, 2 * t->num_scales, hipMemcpyHostToDevice, dev->stream);
+      if (e == hipSuccess) rc = launch_scales_from_wire(stage, t->scales(), t->num_scales, scheme->scale_dtype, dev->stream);
+      dev->release(stage, stage_bytes);  // (stream ordered: the next owner's work queues behind the kernel)
+    }
+  }
   if (e == hipSuccess) e = hipStreamSynchronize(dev->stream);
-  if (e != hipSuccess) {
+  if (e != hipSuccess || rc != BQ_OK) {
     bq_tensor_release(t);
-    BQ_FAIL(BQ_ERR_HIP, "host to device copy failed: %s", hipGetErrorString(e));
+    if (e != hipSuccess) BQ_FAIL(BQ_ERR_HIP, "host to device copy failed: %s", hipGetErrorString(e));
+    return rc;
   }
   *out = t;
   return BQ_OK;
@@ -601,15 +617,28 @@ extern "C" bq_status bq_q_into_data(const bq_tensor* t, uint8_t* bytes, size_t c
   BQ_NOTNULL(t);
   BQ_NOTNULL(len_out);
   if (t->dtype != BQ_QFLOAT) BQ_FAIL(BQ_ERR_DTYPE, "bq_q_into_data on a float tensor");
-  const size_t need = t->value_bytes + 4 * t->num_scales;
+  const size_t ssz = scale_size(t->scheme);
+  const size_t need = t->value_bytes + ssz * t->num_scales;
   *len_out = need;
   if (capacity < need) BQ_FAIL(BQ_ERR_SIZE, "host buffer of %zu bytes for a blob of %zu", capacity, need);
   BQ_NOTNULL(bytes);
   hipStream_t st = t->dev->stream;
   if (t->value_bytes) BQ_HIP(hipMemcpyAsync(bytes, t->data, t->value_bytes, hipMemcpyDeviceToHost, st));
-  BQ_HIP(hipMemcpyAsync(bytes + t->value_bytes, t->scales(), 4 * t->num_scales, hipMemcpyDeviceToHost, st));
-  BQ_HIP(hipStreamSynchronize(st));
-  return BQ_OK;
+  if (ssz == 4) {
+    BQ_HIP(hipMemcpyAsync(bytes + t->value_bytes, t->scales(), 4 * t->num_scales, hipMemcpyDeviceToHost, st));
+    BQ_HIP(hipStreamSynchronize(st));
+    return BQ_OK;
+  }
+  void* stage = nullptr;
+  size_t stage_bytes = 0;
+  BQ_TRY(t->dev->alloc(2 * t->num_scales, &stage, &stage_bytes));
+  bq_status rc = launch_scales_to_wire(t->scales(), stage, t->num_scales, t->scheme.scale_dtype, st);
+  hipError_t e = hipSuccess;
+  if (rc == BQ_OK) e = hipMemcpyAsync(bytes + t->value_bytes, stage, 2 * t->num_scales, hipMemcpyDeviceToHost, st);
+  if (e == hipSuccess) e = hipStreamSynchronize(st);
+  t->dev->release(stage, stage_bytes);
+  if (e != hipSuccess) BQ_FAIL(BQ_ERR_HIP, "device to host copy failed: %s", hipGetErrorString(e));
+  return rc;
 }
 
 // ================================================================================ quantize
@@ -675,13 +704,21 @@ static bq_status quantize_impl(const bq_tensor* x, const bq_scheme* scheme, cons
       return rc;
     }
   }
+  const int sdt = scheme->scale_dtype;
   do {
     if (!dynamic) {
-      hipError_t e = hipMemcpyAsync(q->scales(), scales->data, 4 * q->num_scales, hipMemcpyDeviceToDevice, st);
-      if (e != hipSuccess) {
-        set_error("copying scales failed: %s", hipGetErrorString(e));
-        rc = BQ_ERR_HIP;
-        break;
+      // the stored scale is the given one, rounded up to the scale dtype first (scale_to_dtype,
+      // crates/burn-ndarray/src/ops/qtensor.rs:90-95): the values are divided by what is stored
+      if (sdt == BQ_SCALE_F32) {
+        hipError_t e = hipMemcpyAsync(q->scales(), scales->data, 4 * q->num_scales, hipMemcpyDeviceToDevice, st);
+        if (e != hipSuccess) {
+          set_error("copying scales failed: %s", hipGetErrorString(e));
+          rc = BQ_ERR_HIP;
+          break;
+        }
+      } else {
+        rc = launch_round_scales(static_cast<const float*>(scales->data), q->scales(), q->num_scales, sdt, st);
+        if (rc != BQ_OK) break;
       }
     }
     if (n == 0) break;
@@ -692,20 +729,18 @@ static bq_status quantize_impl(const bq_tensor* x, const bq_scheme* scheme, cons
         uint32_t* cells = reinterpret_cast<uint32_t*>(q->scales() + 1);
         rc = bqk_absmax_f32(xin, n, cells, st);
         if (rc != BQ_OK) break;
-        rc = bqk_quantize_per_tensor_from_absmax(xin, n, cells, q->scales(), scheme->value,
-                                                 scheme->store, q->data, st);
+        rc = launch_quantize_per_tensor(xin, n, reinterpret_cast<const float*>(cells), true, q->scales(), scheme->value,
+                                        scheme->store, q->data, sdt, st);
       } else {
-        rc = bqk_quantize_per_tensor(xin, n, q->scales(), scheme->value, scheme->store, q->data, st);
+        rc = launch_quantize_per_tensor(xin, n, q->scales(), false, nullptr, scheme->value, scheme->store, q->data, sdt, st);
       }
     } else if (run > 0 && fused_block_ok(static_cast<int>(run), scheme->value) && run <= 512) {
-      rc = dynamic ? bqk_quantize_dynamic_block(xin, n, static_cast<int32_t>(run), scheme->value,
-                                                scheme->store, q->data, q->scales(), st)
-                   : bqk_quantize_block(xin, n, static_cast<int32_t>(run), q->scales(), scheme->value,
-                                        scheme->store, q->data, st);
+      rc = launch_quantize_run_block(xin, n, static_cast<int>(run), dynamic ? nullptr : q->scales(), q->scales(),
+                                     scheme->value, scheme->store, q->data, sdt, st);
     } else {
       size_t blk[BQ_MAX_RANK];
       block_dims(*scheme, x->rank, blk);
-      rc = launch_quantize_rect(xin, x->shape, x->rank, blk, scheme->value, scheme->store, dynamic,
+      rc = launch_quantize_rect(xin, x->shape, x->rank, blk, scheme->value, scheme->store, dynamic, sdt,
                                 q->data, q->scales(), st);
     }
   } while (false);

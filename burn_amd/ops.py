@@ -227,11 +227,20 @@ class TensorData:
         return n.value
 
     def split(self):
-        """(values bytes, f32 scales) -- the two regions of the blob."""
-        n_scales = int(np.prod(params_shape(self.shape, self.scheme)))
-        cut = self.bytes.size - 4 * n_scales
-        return self.bytes[:cut], self.bytes[cut:].view(np.float32).reshape(
-            params_shape(self.shape, self.scheme))
+        """(values bytes, scales as f32) -- the two regions of the blob. 2-byte scales (f16 / bf16)
+        are widened exactly (decode_scales, crates/burn-std/src/tensor/quantization.rs:418-441)."""
+        from .quantization import ScaleDtype
+        pshape = params_shape(self.shape, self.scheme)
+        n_scales = int(np.prod(pshape))
+        cut = self.bytes.size - self.scheme.scale_dtype.size() * n_scales
+        raw = self.bytes[cut:]
+        if self.scheme.scale_dtype == ScaleDtype.F32:
+            scales = raw.view(np.float32)
+        elif self.scheme.scale_dtype == ScaleDtype.F16:
+            scales = raw.view(np.float16).astype(np.float32)
+        else:
+            scales = f32_from_bf16_bits(raw.view(np.uint16))
+        return self.bytes[:cut], scales.reshape(pshape)
 
 
 class QTensorOps:

@@ -2,7 +2,8 @@
 
 `QuantScheme` mirrors cubecl_common::quant::scheme::QuantScheme as burn re-exports it
 (crates/burn-std/src/tensor/quantization.rs:4-6), restricted to what this backend implements:
-symmetric Q8S / Q4S values, per-tensor or per-block f32 scales, Native or PackedU32(0) store.
+symmetric Q8S / Q4S values, per-tensor or per-block scales stored as f32, f16 or bf16, Native or
+PackedU32(0) store.
 """
 from __future__ import annotations
 
@@ -31,6 +32,12 @@ class QuantStore(IntEnum):
 
 class ScaleDtype(IntEnum):
     F32 = _lib.SCALE_F32
+    F16 = _lib.SCALE_F16
+    BF16 = _lib.SCALE_BF16
+
+    def size(self) -> int:
+        """scale_size -- crates/burn-std/src/tensor/quantization.rs:409-416."""
+        return 4 if self == ScaleDtype.F32 else 2
 
 
 @dataclass(frozen=True)
@@ -52,8 +59,11 @@ class QuantScheme:
     def per_block(self, block, scale_dtype: ScaleDtype = ScaleDtype.F32) -> "QuantScheme":
         return replace(self, block=tuple(int(b) for b in block), scale_dtype=scale_dtype)
 
-    def per_tensor(self) -> "QuantScheme":
-        return replace(self, block=None)
+    def per_tensor(self, scale_dtype: Optional[ScaleDtype] = None) -> "QuantScheme":
+        return replace(self, block=None, scale_dtype=self.scale_dtype if scale_dtype is None else scale_dtype)
+
+    def with_scale_dtype(self, scale_dtype: ScaleDtype) -> "QuantScheme":
+        return replace(self, scale_dtype=scale_dtype)
 
     def num_quants(self) -> int:
         return 32 // self.value.size_bits() if self.store == QuantStore.PackedU32 else 1

@@ -56,7 +56,10 @@ enum { BQ_F32 = 0, BQ_BF16 = 1, BQ_QFLOAT = 2 };
 enum { BQ_Q8S = 0, BQ_Q4S = 1 };
 enum { BQ_LEVEL_TENSOR = 0, BQ_LEVEL_BLOCK = 1 };
 enum { BQ_STORE_NATIVE = 0, BQ_STORE_PACKED_U32 = 1 };
-enum { BQ_SCALE_F32 = 0 };
+/* ScaleDtype. F16 / BF16: the quantizer divides by the scale rounded UP to the scale dtype
+ * (scale_to_dtype, crates/burn-std/src/tensor/quantization.rs:354-368) and the blob stores 2 bytes
+ * per scale (encode_scales, same file). */
+enum { BQ_SCALE_F32 = 0, BQ_SCALE_F16 = 1, BQ_SCALE_BF16 = 2 };
 
 /* The fields of QuantScheme this path reads. `block` holds block_rank extents aligned to the
  * trailing dims (BlockSize::to_dim_vec pads the leading dims with 1). PackedU32 always packs
@@ -65,7 +68,7 @@ typedef struct bq_scheme {
   uint8_t value;       /* BQ_Q8S | BQ_Q4S */
   uint8_t level;       /* BQ_LEVEL_TENSOR | BQ_LEVEL_BLOCK */
   uint8_t store;       /* BQ_STORE_NATIVE (Q8S only) | BQ_STORE_PACKED_U32 */
-  uint8_t scale_dtype; /* BQ_SCALE_F32 */
+  uint8_t scale_dtype; /* BQ_SCALE_F32 | BQ_SCALE_F16 | BQ_SCALE_BF16 */
   uint8_t block_rank;
   uint8_t reserved[3];
   uint8_t block[BQ_MAX_RANK];

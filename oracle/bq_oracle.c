@@ -453,3 +453,90 @@ int bqo_dequantize_mt(const int8_t* q, const size_t* shape, int rank, const bqo_
   }
   return 0;
 }
+
+/* ---- scale dtypes --------------------------------------------------------------------------- */
+static uint32_t f32_bits(float f) { uint32_t u; memcpy(&u, &f, 4); return u; }
+static float bits_f32(uint32_t u) { float f; memcpy(&f, &u, 4); return f; }
+
+/* f32 -> f16, round to nearest even (what half::f16::from_f32 does) */
+static uint16_t f16_from_f32_rne(float f) {
+  const uint32_t u = f32_bits(f), sign = (u >> 16) & 0x8000u, mag = u & 0x7FFFFFFFu;
+  if (mag > 0x7F800000u) return (uint16_t)(sign | 0x7E00u);
+  if (mag >= 0x477FF000u) return (uint16_t)(sign | 0x7C00u);           /* >= 65520 rounds to infinity */
+  if (mag < 0x33000001u) return (uint16_t)sign;                          /* <= 2^-25 rounds to zero */
+  int e = (int)(mag >> 23) - 127;
+  uint32_t man = (mag & 0x7FFFFFu) | 0x800000u;                          /* 24-bit significand */
+  int shift = e < -14 ? 13 + (-14 - e) : 13;                             /* bits dropped */
+  uint32_t kept = man >> shift, rest = man & ((1u << shift) - 1u), half = 1u << (shift - 1);
+  if (rest > half || (rest == half && (kept & 1u))) ++kept;
+  if (e < -14) return (uint16_t)(sign | kept);                           /* subnormal (a carry makes it 2^-14) */
+  return (uint16_t)(sign | (((uint32_t)(e + 15) << 10) + (kept - 0x400u)));  /* a carry bumps the exponent */
+}
+
+static float f32_from_f16(uint16_t h) {
+  const uint32_t sign = ((uint32_t)h & 0x8000u) << 16, ex = (h >> 10) & 0x1Fu, man = h & 0x3FFu;
+  if (ex == 0) {
+    float t = (float)man * 5.9604644775390625e-8f; /* man * 2^-24 */
+    return bits_f32(sign | f32_bits(t));
+  }
+  if (ex == 31) return bits_f32(sign | 0x7F800000u | (man << 13));
+  return bits_f32(sign | ((ex + 112u) << 23) | (man << 13));
+}
+
+static uint16_t bf16_from_f32_rne(float f) {
+  uint32_t u = f32_bits(f);
+  if ((u & 0x7FFFFFFFu) > 0x7F800000u) return (uint16_t)((u >> 16) | 0x40u);
+  u += 0x7FFFu + ((u >> 16) & 1u);
+  return (uint16_t)(u >> 16);
+}
+
+float bqo_scale_to_dtype(float scale, int dtype) {
+  if (dtype == BQO_SCALE_F32) return scale;
+  if (scale != scale || scale == INFINITY || scale == -INFINITY) return scale;
+  /* start from the nearest representable value, step up while it is below the scale */
+  if (dtype == BQO_SCALE_F16) {
+    uint16_t h = f16_from_f32_rne(scale);
+    float back = f32_from_f16(h);
+    if (back < scale) {                      /* next representable value toward +infinity */
+      if (h & 0x8000u) h = (uint16_t)((h & 0x7FFFu) == 0 ? 0x0001u : h - 1u); else h = (uint16_t)(h + 1u);
+      back = f32_from_f16(h);
+    }
+    if (back == INFINITY) back = 65504.0f;   /* a finite scale saturates (parity unpinned) */
+    if (back == -INFINITY) back = -65504.0f; /* (RNE of a finite value below -65504; -65504 is no smaller) */
+    return back;
+  }
+  uint16_t b = bf16_from_f32_rne(scale);
+  float back = bits_f32((uint32_t)b << 16);
+  if (back < scale) {
+    if (b & 0x8000u) b = (uint16_t)((b & 0x7FFFu) == 0 ? 0x0001u : b - 1u); else b = (uint16_t)(b + 1u);
+    back = bits_f32((uint32_t)b << 16);
+  }
+  if (back == INFINITY) back = bits_f32(0x7F7F0000u);
+  if (back == -INFINITY) back = bits_f32(0xFF7F0000u);
+  return back;
+}
+
+size_t bqo_scale_size(int dtype) { return dtype == BQO_SCALE_F32 ? 4 : 2; }
+
+void bqo_encode_scales(const float* scales, size_t n, int dtype, uint8_t* out) {
+  for (size_t i = 0; i < n; ++i) {
+    if (dtype == BQO_SCALE_F32) {
+      memcpy(out + 4 * i, scales + i, 4);
+    } else {
+      uint16_t h = dtype == BQO_SCALE_F16 ? f16_from_f32_rne(scales[i]) : bf16_from_f32_rne(scales[i]);
+      memcpy(out + 2 * i, &h, 2);
+    }
+  }
+}
+
+void bqo_decode_scales(const uint8_t* in, size_t n, int dtype, float* out) {
+  for (size_t i = 0; i < n; ++i) {
+    if (dtype == BQO_SCALE_F32) {
+      memcpy(out + i, in + 4 * i, 4);
+    } else {
+      uint16_t h;
+      memcpy(&h, in + 2 * i, 2);
+      out[i] = dtype == BQO_SCALE_F16 ? f32_from_f16(h) : bits_f32((uint32_t)h << 16);
+    }
+  }
+}

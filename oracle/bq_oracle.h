@@ -22,6 +22,18 @@
  *   bqo_encode/decode    burn-std/src/tensor/quantization.rs:605-625, tests .../quantization/data.rs:6-50
  *   bqo_block_of         ops/quantize.rs:171-206 + brute force against a reshape on small shapes
  *   bqo_q_matmul         ops/matmul.rs:141-168, :204-249 (known 3x4 and 3x16 products)
+ *   bqo_scale_to_dtype   f32 / f16 / bf16. The rule is the reference's doc comment (burn-std
+ *                        .../quantization.rs:354-368: "the smallest value representable by the scale
+ *                        dtype that is no smaller"); its arithmetic lives in cubecl-common (absent).
+ *                        For IEEE f16 / bf16 the rule fixes the result: checked by brute force over
+ *                        all 65 536 patterns of each format (representable values are fixed points,
+ *                        the f32 neighbour above goes to the next representable value, the one
+ *                        below stays) and by the reference test's own scales and properties
+ *                        (:631-657: rounded >= scale, the codec leaves a rounded scale alone).
+ *                        PARITY UNPINNED: what a finite scale beyond the dtype's largest finite
+ *                        value becomes (this restatement saturates to it, as the reference's test
+ *                        comment says of e4m3), and UE4M3 / UE8M0 (not implemented).
+ *   bqo_encode/decode_scales  same test (:631-657) and the two-level layout test (:659-684).
  */
 #ifndef BQ_ORACLE_H
 #define BQ_ORACLE_H
@@ -38,6 +50,7 @@ extern "C" {
 enum { BQO_Q8S = 0, BQO_Q4S = 1 };            /* QuantValue (symmetric signed ints only) */
 enum { BQO_LEVEL_TENSOR = 0, BQO_LEVEL_BLOCK = 1 };
 enum { BQO_STORE_NATIVE = 0, BQO_STORE_PACKED_U32 = 1 };
+enum { BQO_SCALE_F32 = 0, BQO_SCALE_F16 = 1, BQO_SCALE_BF16 = 2 };   /* ScaleDtype */
 
 /* Mirrors the fields of cubecl_common::quant::scheme::QuantScheme that this path reads. */
 typedef struct {
@@ -96,6 +109,16 @@ void bqo_matmul_f32(const float* a, const float* b, float* c, size_t m, size_t k
 /* q_matmul with a float lhs and a quantized rhs: dequantize(rhs) -> f32 matmul. */
 int bqo_q_matmul(const float* lhs, size_t m, const int8_t* rhs_q, const size_t* rhs_shape,
                  const bqo_scheme* s, const float* rhs_scales, float* out);
+
+/* scale_to_dtype (burn-std/src/tensor/quantization.rs:354-368): the smallest value the scale dtype
+ * represents that is no smaller than `scale`. NdArray::quantize applies it to every scale before
+ * dividing (burn-ndarray/src/ops/qtensor.rs:90-95). */
+float bqo_scale_to_dtype(float scale, int dtype);
+/* scale_size / encode_scales / decode_scales (same file, :409-464): bytes per scale on the wire;
+ * f16 and bf16 are written with round-to-nearest-even (half::from_f32), native endian. */
+size_t bqo_scale_size(int dtype);
+void bqo_encode_scales(const float* scales, size_t n, int dtype, uint8_t* out);
+void bqo_decode_scales(const uint8_t* in, size_t n, int dtype, float* out);
 
 /* Threads used by the *_mt variants below (OpenMP), 1 when built without it. */
 int bqo_max_threads(void);

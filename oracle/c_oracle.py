@@ -95,6 +95,14 @@ def lib():
         L.bqo_matmul_f32.restype = None
         L.bqo_q_matmul.argtypes = [pf, sz, pi8, psz, ps, pf, pf]
         L.bqo_max_threads.restype = i32
+        L.bqo_scale_to_dtype.argtypes = [C.c_float, i32]
+        L.bqo_scale_to_dtype.restype = C.c_float
+        L.bqo_scale_size.argtypes = [i32]
+        L.bqo_scale_size.restype = sz
+        L.bqo_encode_scales.argtypes = [pf, sz, i32, pu8]
+        L.bqo_encode_scales.restype = None
+        L.bqo_decode_scales.argtypes = [pu8, sz, i32, pf]
+        L.bqo_decode_scales.restype = None
         _lib = L
     return _lib
 
@@ -260,3 +268,35 @@ def q_matmul(lhs, rhs_q, scheme, rhs_scales):
 
 def max_threads():
     return lib().bqo_max_threads()
+
+
+SCALE_F32, SCALE_F16, SCALE_BF16 = 0, 1, 2
+
+
+def scale_to_dtype(scales, dtype):
+    """scale_to_dtype applied to every entry (burn-ndarray/src/ops/qtensor.rs:90-95)."""
+    a = np.ascontiguousarray(scales, dtype=np.float32)
+    f = lib().bqo_scale_to_dtype
+    return np.array([f(float(v), dtype) for v in a.reshape(-1)], np.float32).reshape(a.shape)
+
+
+def encode_scales(scales, dtype):
+    a = np.ascontiguousarray(scales, dtype=np.float32).reshape(-1)
+    out = np.empty(a.size * lib().bqo_scale_size(dtype), np.uint8)
+    lib().bqo_encode_scales(_p(a, C.c_float), a.size, dtype, _p(out, C.c_uint8))
+    return out
+
+
+def decode_scales(data, dtype):
+    d = np.ascontiguousarray(data, dtype=np.uint8)
+    n = d.size // lib().bqo_scale_size(dtype)
+    out = np.empty(n, np.float32)
+    lib().bqo_decode_scales(_p(d, C.c_uint8), n, dtype, _p(out, C.c_float))
+    return out
+
+
+def encode_with_scale_dtype(q, scheme, scales, dtype):
+    """The QuantizedBytes blob with the scales region written in `dtype`: values || encoded scales."""
+    blob = encode(q, scheme, np.zeros_like(np.ascontiguousarray(scales, np.float32)))
+    n = int(np.ascontiguousarray(scales).size)
+    return np.concatenate([blob[: blob.size - 4 * n], encode_scales(scales, dtype)])

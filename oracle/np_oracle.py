@@ -154,3 +154,32 @@ def q_permute(q, scales, block, axes):
 def q_flip(q, scales, axes):
     """NdArray q_flip (qtensor.rs:338-347): the values are flipped, the parameters kept."""
     return np.flip(np.asarray(q), axis=tuple(axes)).copy(), np.asarray(scales, np.float32)
+
+
+def scale_to_dtype(scales, dtype="F32"):
+    """scale_to_dtype (crates/burn-std/src/tensor/quantization.rs:354-368): smallest value of the
+    scale dtype that is no smaller. A second, independent restatement: numpy's own f16 conversion
+    (round to nearest even) stepped up with nextafter where it fell below; bf16 through bit masks.
+    A finite value past the largest finite one saturates to it."""
+    s = np.asarray(scales, np.float32)
+    if dtype == "F32":
+        return s.copy()
+    if dtype == "F16":
+        with np.errstate(over="ignore"):
+            h = s.astype(np.float16)
+            below = h.astype(np.float32) < s
+            h = np.where(below, np.nextafter(h, np.float16(np.inf)), h)
+        out = h.astype(np.float32)
+        big = np.float32(65504.0)
+        out = np.where(np.isfinite(s) & (out == np.inf), big, out)
+        return np.where(np.isfinite(s) & (out == -np.inf), -big, out).astype(np.float32)
+    if dtype == "BF16":
+        u = s.view(np.uint32).astype(np.uint64)
+        low = u & 0xFFFF
+        neg = (u >> 31) == 1
+        up = np.where(neg, u & 0xFFFF0000, (u + 0xFFFF) & 0xFFFF0000)
+        r = np.where(low == 0, u, up)
+        r = np.where(np.isfinite(s) & ((r & 0x7FFFFFFF) >= 0x7F800000), (r & 0x80000000) | 0x7F7F0000, r)
+        r = np.where(np.isfinite(s), r, u)
+        return r.astype(np.uint32).view(np.float32)
+    raise ValueError(dtype)

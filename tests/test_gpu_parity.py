@@ -16,6 +16,7 @@ pytestmark = pytest.mark.gpu
 
 import burn_amd as ba  # noqa: E402
 from burn_amd import FloatOps, QTensorOps, QuantScheme, QuantStore, QuantValue, TensorData  # noqa: E402
+from burn_amd.quantization import ScaleDtype  # noqa: E402
 
 VAL = {QuantValue.Q8S: (co.Q8S, "Q8S"), QuantValue.Q4S: (co.Q4S, "Q4S")}
 
@@ -577,6 +578,82 @@ def test_validate_mode_fails_where_the_reference_panics(dev):
         dev.set_validate(False)
     QTensorOps.quantize_dynamic(FloatOps.float_from_data(bad_nan, dev), scheme)  # unspecified integers, no error
     dev.sync()
+
+
+# ------------------------------------------------------------------ f16 / bf16 scales
+
+SDT = {ScaleDtype.F16: (co.SCALE_F16, "F16"), ScaleDtype.BF16: (co.SCALE_BF16, "BF16")}
+
+
+def check_scale_dtype(dev, x, scheme, given_scales=None):
+    """quantize / quantize_dynamic with 2-byte scales against the oracle composed the way
+    burn-ndarray composes it (qtensor.rs:90-95): range -> q_params -> scale_to_dtype -> quantize
+    against the rounded scale; the blob carries the scales encoded in the scale dtype."""
+    code, _ = SDT[scheme.scale_dtype]
+    osch = oscheme(scheme)
+    if given_scales is None:
+        lo, hi = co.compute_range(x, osch)
+        raw = co.compute_q_params(lo, hi, osch.value)
+        tq = QTensorOps.quantize_dynamic(FloatOps.float_from_data(x, dev), scheme)
+    else:
+        raw = np.ascontiguousarray(given_scales, np.float32)
+        tq = QTensorOps.quantize(FloatOps.float_from_data(x, dev), scheme, FloatOps.float_from_data(raw, dev))
+    s_ref = co.scale_to_dtype(raw, code)
+    q_ref = co.quantize(x, osch, s_ref)
+    blob = QTensorOps.q_into_data(tq)
+    assert blob.bytes.size == TensorData.data_len(x.shape, scheme)
+    assert blob.bytes.tobytes() == co.encode_with_scale_dtype(q_ref, osch, s_ref, code).tobytes(), "blob differs"
+    q_gpu, s_gpu = unpack_blob(blob)
+    assert s_gpu.reshape(-1).tobytes() == np.ascontiguousarray(s_ref, np.float32).reshape(-1).tobytes()
+    assert (q_gpu == q_ref).all()
+    d_ref = co.dequantize(q_ref, osch, s_ref)
+    assert FloatOps.float_into_data(QTensorOps.dequantize(tq)).tobytes() == d_ref.tobytes()
+    # save / load: the blob loads back to the same tensor (one H2D copy of values, scales widened)
+    again = QTensorOps.q_from_data(blob, dev)
+    assert QTensorOps.q_into_data(again).bytes.tobytes() == blob.bytes.tobytes()
+    assert FloatOps.float_into_data(QTensorOps.dequantize(again)).tobytes() == d_ref.tobytes()
+    return tq, q_ref, s_ref
+
+
+@pytest.mark.parametrize("sdt", [ScaleDtype.F16, ScaleDtype.BF16])
+@pytest.mark.parametrize("value", [QuantValue.Q8S, QuantValue.Q4S])
+@pytest.mark.parametrize("block", [None, (32,), (16,), (2, 32)])
+def test_quantize_with_two_byte_scales(dev, sdt, value, block):
+    x = awkward((48, 256), 21)
+    scheme = QuantScheme(value=value, scale_dtype=sdt) if block is None else QuantScheme(value=value).per_block(block, sdt)
+    check_scale_dtype(dev, x, scheme)
+    if value == QuantValue.Q8S:
+        native = QuantScheme(store=QuantStore.Native, scale_dtype=sdt) if block is None else \
+            QuantScheme(store=QuantStore.Native).per_block(block, sdt)
+        check_scale_dtype(dev, x, native)
+    # given scales that the dtype does not represent: rounded up before anything is divided
+    n = int(np.prod(ba.quantization.params_shape(x.shape, scheme)))
+    given = np.random.default_rng(3).uniform(0.01, 0.2, n).astype(np.float32)
+    given[:: 7] = 0.0           # zero scales stay zero (and quantize against 0.1)
+    check_scale_dtype(dev, x, scheme, given_scales=given)
+
+
+@pytest.mark.parametrize("sdt", [ScaleDtype.F16, ScaleDtype.BF16])
+def test_two_byte_scales_over_the_exponent_range(dev, sdt):
+    """Blocks whose scale runs from far below the format's subnormals to past its largest value."""
+    rng = np.random.default_rng(12)
+    exps = np.arange(-40, 30)
+    x = np.ldexp(rng.standard_normal((len(exps), 64)), exps[:, None]).astype(np.float32)
+    check_scale_dtype(dev, x, QuantScheme().per_block((32,), sdt))
+    check_scale_dtype(dev, x[20], QuantScheme(store=QuantStore.Native, scale_dtype=sdt))
+
+
+@pytest.mark.parametrize("sdt", [ScaleDtype.F16, ScaleDtype.BF16])
+def test_q_matmul_with_two_byte_scales(dev, sdt):
+    rng = np.random.default_rng(8)
+    w = (rng.standard_normal((512, 384)) * 0.02).astype(np.float32)
+    scheme = QuantScheme().per_block((32,), sdt)
+    tw, q_ref, s_ref = check_scale_dtype(dev, w, scheme)
+    for m in (1, 16, 80):
+        x = rng.standard_normal((m, 512)).astype(np.float32)
+        out = FloatOps.float_into_data(QTensorOps.q_matmul(FloatOps.float_from_data(x, dev), tw))
+        ref = no.q_matmul_f64(x, q_ref, s_ref, [32])
+        matmul_check(out, ref)
 
 
 # ------------------------------------------------------------------ the configs at full size

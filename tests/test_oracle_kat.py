@@ -334,3 +334,51 @@ def test_c_and_numpy_restatements_agree(value, block):
     words = co.pack_u32(qc, sch.value)
     assert words.tobytes() == no.pack_u32(qn, value).tobytes()
     assert (co.unpack_u32(words, x.shape, sch.value) == qc).all()
+
+
+# ------------------------------------------------------------------ scale dtypes (f16 / bf16)
+
+def _all_finite_patterns(kind):
+    bits = np.arange(65536, dtype=np.uint32).astype(np.uint16)
+    vals = bits.view(np.float16).astype(np.float32) if kind == "F16" else (bits.astype(np.uint32) << 16).view(np.float32)
+    vals = vals[np.isfinite(vals)]
+    return np.unique(vals)          # ascending, -0.0 and 0.0 merged
+
+
+@pytest.mark.parametrize("kind,code", [("F16", co.SCALE_F16), ("BF16", co.SCALE_BF16)])
+def test_scale_to_dtype_is_the_ceiling_onto_the_format(kind, code):
+    """"The smallest value representable by the scale dtype that is no smaller" fixes the function
+    for an IEEE format. Brute force over every finite value of the format: it is a fixed point,
+    the f32 just above it maps to the next value of the format, the f32 just below maps to itself.
+    Both restatements (C, numpy) must pass, and agree on random scales."""
+    grid = _all_finite_patterns(kind)
+    up = np.nextafter(grid, np.float32(np.inf)).astype(np.float32)
+    down = np.nextafter(grid, np.float32(-np.inf)).astype(np.float32)
+    nxt = np.concatenate([grid[1:], grid[-1:]])          # past the largest finite value: saturates
+    for f in (lambda a: no.scale_to_dtype(a, kind), lambda a: co.scale_to_dtype(a, code)):
+        assert (f(grid).view(np.uint32) == grid.view(np.uint32)).all() or (f(grid) == grid).all()
+        assert (f(up)[:-1] == nxt[:-1]).all()
+        assert f(up)[-1] == grid[-1]
+        assert (f(down)[1:] == grid[1:]).all()
+        assert f(down)[0] == grid[0]                       # below the most negative value: that value is no smaller
+    rng = np.random.default_rng(31)
+    s = np.ldexp(rng.standard_normal(20000), rng.integers(-30, 18, 20000)).astype(np.float32)
+    assert (no.scale_to_dtype(s, kind) == co.scale_to_dtype(s, code)).all()
+    inside = s <= grid[-1]      # past the largest finite value a scale saturates instead (parity unpinned there)
+    assert (no.scale_to_dtype(s, kind)[inside] >= s[inside]).all()
+    assert (no.scale_to_dtype(s, kind)[~inside] == grid[-1]).all()
+
+
+def test_scale_to_dtype_survives_the_codec_like_the_reference_test():
+    """crates/burn-std/src/tensor/quantization.rs:626-657 (`scale_to_dtype_survives_the_codec`) with
+    its own scales: encoding a rounded scale must not move it, and rounding never goes down."""
+    scales = np.float32([0.5, 0.3, 1.0 / 3.0, 500.0, 1e-3, 7.7e-4])
+    for code in (co.SCALE_F32, co.SCALE_F16, co.SCALE_BF16):
+        rounded = co.scale_to_dtype(scales, code)
+        via_codec = co.decode_scales(co.encode_scales(rounded, code), code)
+        assert (rounded == via_codec).all()
+        assert (rounded >= scales).all()
+    assert co.encode_scales(scales, co.SCALE_F16).size == 12 and co.encode_scales(scales, co.SCALE_F32).size == 24
+    # exactly representable values pin the byte layout (as in the reference's two-level layout test)
+    assert co.encode_scales(np.float32([0.5, 0.125]), co.SCALE_F16).view(np.uint16).tolist() == [0x3800, 0x3000]
+    assert co.encode_scales(np.float32([0.5, 0.125]), co.SCALE_BF16).view(np.uint16).tolist() == [0x3F00, 0x3E00]
