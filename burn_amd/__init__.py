@@ -9,11 +9,12 @@ Importing the package does not load the library; the first operation does, and f
 the shared object has not been built (`python -m burn_amd.build`).
 """
 from ._lib import BF16, F32, QFLOAT, BurnqError
-from .ops import Device, FloatOps, ModuleOps, QTensorOps, Tensor, TensorData, bf16_bits_from_f32, f32_from_bf16_bits
+from .ops import (Device, FloatOps, ModuleOps, PackReader, PackWriter, QTensorOps, Tensor, TensorData, bf16_bits_from_f32,
+                  f32_from_bf16_bits)
 from .quantization import QuantScheme, QuantStore, QuantValue, ScaleDtype, params_shape
 
 __all__ = [
-    "BF16", "F32", "QFLOAT", "BurnqError", "Device", "FloatOps", "ModuleOps", "QTensorOps", "Tensor",
+    "BF16", "F32", "QFLOAT", "BurnqError", "Device", "FloatOps", "ModuleOps", "PackReader", "PackWriter", "QTensorOps", "Tensor",
     "TensorData", "QuantScheme", "QuantStore", "QuantValue", "ScaleDtype", "params_shape",
     "bf16_bits_from_f32", "f32_from_bf16_bits",
 ]

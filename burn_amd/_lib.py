@@ -40,6 +40,27 @@ class CScheme(C.Structure):
     ]
 
 
+class CPackEntry(C.Structure):
+    """bq_pack_entry"""
+
+    _fields_ = [
+        ("name", C.c_char_p),
+        ("dtype", C.c_int32),
+        ("rank", C.c_int32),
+        ("shape", C.c_size_t * MAX_RANK),
+        ("data_begin", C.c_uint64),
+        ("data_end", C.c_uint64),
+        ("has_param_id", C.c_int32),
+        ("param_id", C.c_uint64),
+        ("has_scheme", C.c_int32),
+        ("scheme", CScheme),
+        ("data", C.c_void_p),
+    ]
+
+
+PACK_DTYPES = ["F64", "F32", "Flex32", "F16", "BF16", "I64", "I32", "I16", "I8", "U64", "U32", "U16", "U8", "Bool", "QFloat"]
+PACK_F32, PACK_BF16, PACK_QFLOAT = 1, 4, 14
+
 _vp, _sz, _i32 = C.c_void_p, C.c_size_t, C.c_int32
 _psz = C.POINTER(C.c_size_t)
 _pvp = C.POINTER(C.c_void_p)
@@ -106,6 +127,23 @@ SIGNATURES = {
                             _sz, _vp]),
     "bqk_q_linear": (_i32, [_vp, _i32, _sz, _sz, _sz, _vp, _vp, _i32, _i32, _i32, _vp, _i32, _vp, _vp,
                             _sz, _vp]),
+    "bq_pack_data_section_start": (_sz, [_sz]),
+    "bq_pack_open": (_i32, [C.c_char_p, _pvp]),
+    "bq_pack_from_bytes": (_i32, [_vp, _sz, _i32, _pvp]),
+    "bq_pack_close": (_i32, [_vp]),
+    "bq_pack_num_tensors": (C.c_int64, [_vp]),
+    "bq_pack_entry_at": (_i32, [_vp, C.c_int64, C.POINTER(CPackEntry)]),
+    "bq_pack_find": (_i32, [_vp, C.c_char_p, C.POINTER(CPackEntry)]),
+    "bq_pack_metadata": (C.c_char_p, [_vp, C.c_char_p]),
+    "bq_pack_load": (_i32, [_vp, C.c_char_p, _ps, _vp, _pvp]),
+    "bq_pack_writer_new": (_i32, [_pvp]),
+    "bq_pack_writer_free": (_i32, [_vp]),
+    "bq_pack_writer_set_metadata": (_i32, [_vp, C.c_char_p, C.c_char_p]),
+    "bq_pack_writer_add_bytes": (_i32, [_vp, C.c_char_p, _i32, _ps, _psz, _i32, _vp, _sz, _i32, C.c_uint64]),
+    "bq_pack_writer_add_tensor": (_i32, [_vp, C.c_char_p, _vp, _i32, C.c_uint64]),
+    "bq_pack_writer_size": (_i32, [_vp, _psz]),
+    "bq_pack_writer_write_into": (_i32, [_vp, _vp, _sz, _psz]),
+    "bq_pack_writer_write_file": (_i32, [_vp, C.c_char_p]),
     "bqk_q_linear_static": (_i32, [_vp, _i32, _sz, _sz, _sz, _vp, _vp, _i32, _i32, _i32, _vp, _i32, _vp, _vp]),
 }
 STATIC_SCRATCH_BYTES = 16 << 20

@@ -29,6 +29,7 @@ COMMON = [
 # their results are compared bit for bit with a CPU that rounds every operation.
 SOURCES = [
     ("runtime.cpp", ["-x", "hip"]),
+    ("pack.cpp", ["-x", "hip"]),
     ("quantize.hip", ["-ffp-contract=off"]),
     ("dequantize.hip", ["-ffp-contract=off"]),
     ("qmatmul.hip", ["-ffp-contract=off"]),

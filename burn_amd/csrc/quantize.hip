@@ -462,18 +462,17 @@ bq_status launch_count_nonfinite(const float* x, size_t n, uint32_t* counts, hip
   return BQ_OK;
 }
 
-// Plain streaming copy, 16 bytes per lane, 4 chunks per workgroup pass: the known-traffic
-// kernel the HBM counters are calibrated against.
+// Plain streaming copy: the known-traffic kernel the HBM counters are calibrated against, and the
+// ceiling the streaming kernels are compared with. One 16-byte chunk per lane, 256 lanes per
+// workgroup, non-temporal both ways: the best of the shapes measured on a 256 MiB copy (chunks per
+// lane 1 / 2 / 4 / 8 at 256 threads: 6.51 / 6.12 / 6.18 / 4.29 TB/s; 1024 threads x 1: 6.45; 32
+// contiguous bytes per lane: 4.0-5.1; persistent grids of 256-8192 workgroups with the next
+// chunk's loads in flight: 5.5-6.3; plain instead of non-temporal accesses: 5.6; hipMemcpyAsync
+// device to device: 5.4).
 __global__ void __launch_bounds__(256) copy16_kernel(const vuint4* __restrict__ src, vuint4* __restrict__ dst,
                                                      size_t chunks) {
-  const size_t base = static_cast<size_t>(blockIdx.x) * 1024 + threadIdx.x;
-  vuint4 v[4];
-#pragma unroll
-  for (int u = 0; u < 4; ++u)
-    if (base + u * 256 < chunks) v[u] = __builtin_nontemporal_load(src + base + u * 256);
-#pragma unroll
-  for (int u = 0; u < 4; ++u)
-    if (base + u * 256 < chunks) __builtin_nontemporal_store(v[u], dst + base + u * 256);
+  const size_t i = static_cast<size_t>(blockIdx.x) * 256 + threadIdx.x;
+  if (i < chunks) __builtin_nontemporal_store(__builtin_nontemporal_load(src + i), dst + i);
 }
 
 bq_status launch_quantize_rect(const float* x, const size_t* shape, int rank, const size_t* blk,
@@ -801,7 +800,8 @@ extern "C" bq_status bqk_copy(const void* src, void* dst, size_t bytes, void* st
     BQ_FAIL(BQ_ERR_SHAPE, "bqk_copy needs 16-byte aligned pointers and a multiple of 16 bytes");
   if (bytes == 0) return BQ_OK;
   const size_t chunks = bytes / 16;
-  hipLaunchKernelGGL(copy16_kernel, dim3(static_cast<unsigned>((chunks + 1023) / 1024)), dim3(256), 0,
+  if ((chunks + 255) / 256 > 0x7FFFFFFFull) BQ_FAIL(BQ_ERR_SIZE, "bqk_copy: %zu bytes is more than one launch copies", bytes);
+  hipLaunchKernelGGL(copy16_kernel, dim3(static_cast<unsigned>((chunks + 255) / 256)), dim3(256), 0,
                      static_cast<hipStream_t>(stream), static_cast<const vuint4*>(src),
                      static_cast<vuint4*>(dst), chunks);
   BQ_HIP(hipGetLastError());

@@ -588,8 +588,20 @@ extern "C" bq_status bq_q_from_data(bq_device* dev, const uint8_t* bytes, size_t
     BQ_FAIL(BQ_ERR_NULL, "bq_q_from_data: null bytes");
   }
   hipError_t e = hipSuccess;
-  if (t->value_bytes) e = hipMemcpyAsync(t->data, bytes, t->value_bytes, hipMemcpyHostToDevice, dev->stream);
   bq_status rc = BQ_OK;
+  if (ssz == 4 && t->scales_offset == t->value_bytes) {
+    // the device layout is the wire layout (values of a multiple of 256 bytes, f32 scales right
+    // behind them): the whole blob arrives with one copy
+    e = hipMemcpyAsync(t->data, bytes, need, hipMemcpyHostToDevice, dev->stream);
+    if (e == hipSuccess) e = hipStreamSynchronize(dev->stream);
+    if (e != hipSuccess) {
+      bq_tensor_release(t);
+      BQ_FAIL(BQ_ERR_HIP, "host to device copy failed: %s", hipGetErrorString(e));
+    }
+    *out = t;
+    return BQ_OK;
+  }
+  if (t->value_bytes) e = hipMemcpyAsync(t->data, bytes, t->value_bytes, hipMemcpyHostToDevice, dev->stream);
   if (e == hipSuccess && ssz == 4) {
     e = hipMemcpyAsync(t->scales(), bytes + t->value_bytes, 4 * t->num_scales, hipMemcpyHostToDevice, dev->stream);
   } else if (e == hipSuccess) {
@@ -623,6 +635,11 @@ extern "C" bq_status bq_q_into_data(const bq_tensor* t, uint8_t* bytes, size_t c
   if (capacity < need) BQ_FAIL(BQ_ERR_SIZE, "host buffer of %zu bytes for a blob of %zu", capacity, need);
   BQ_NOTNULL(bytes);
   hipStream_t st = t->dev->stream;
+  if (ssz == 4 && t->scales_offset == t->value_bytes) {  // dense on the device as on the wire: one copy
+    BQ_HIP(hipMemcpyAsync(bytes, t->data, need, hipMemcpyDeviceToHost, st));
+    BQ_HIP(hipStreamSynchronize(st));
+    return BQ_OK;
+  }
   if (t->value_bytes) BQ_HIP(hipMemcpyAsync(bytes, t->data, t->value_bytes, hipMemcpyDeviceToHost, st));
   if (ssz == 4) {
     BQ_HIP(hipMemcpyAsync(bytes + t->value_bytes, t->scales(), 4 * t->num_scales, hipMemcpyDeviceToHost, st));

@@ -349,3 +349,101 @@ class ModuleOps:
         check(lib().bq_q_linear(input.handle, weight.handle, bias.handle if bias is not None else None,
                                 -1 if out_dtype is None else out_dtype, C.byref(h)))
         return _wrap(h, input.device)
+
+
+class PackReader:
+    """burn-pack's `Reader` over a .bpk container (crates/burn-pack/src/reader.rs): header and
+    metadata are parsed, the file stays memory-mapped, tensors load straight into device memory."""
+
+    def __init__(self, source):
+        h = C.c_void_p()
+        if isinstance(source, (bytes, bytearray, np.ndarray)):
+            self._keep = np.frombuffer(bytes(source), np.uint8) if not isinstance(source, np.ndarray) else np.ascontiguousarray(source, np.uint8)
+            check(lib().bq_pack_from_bytes(self._keep.ctypes.data, self._keep.size, 0, C.byref(h)))
+        else:
+            check(lib().bq_pack_open(str(source).encode(), C.byref(h)))
+        self.handle = h
+
+    def close(self):
+        h, self.handle = getattr(self, "handle", None), None
+        if h:
+            lib().bq_pack_close(h)
+
+    __del__ = close
+
+    def __len__(self):
+        return lib().bq_pack_num_tensors(self.handle)
+
+    def _entry(self, e):
+        scheme = QuantScheme.from_c(e.scheme) if e.has_scheme else None
+        return {"name": e.name.decode(), "dtype": _lib.PACK_DTYPES[e.dtype], "shape": tuple(e.shape[i] for i in range(e.rank)),
+                "data_offsets": (e.data_begin, e.data_end), "param_id": e.param_id if e.has_param_id else None,
+                "scheme": scheme, "data_ptr": e.data}
+
+    def entries(self):
+        out = []
+        for i in range(len(self)):
+            e = _lib.CPackEntry()
+            check(lib().bq_pack_entry_at(self.handle, i, C.byref(e)))
+            out.append(self._entry(e))
+        return out
+
+    def find(self, name):
+        e = _lib.CPackEntry()
+        check(lib().bq_pack_find(self.handle, name.encode(), C.byref(e)))
+        return self._entry(e)
+
+    def metadata(self, key):
+        v = lib().bq_pack_metadata(self.handle, key.encode())
+        return v.decode() if v is not None else None
+
+    def load(self, name, device: Device, scheme: Optional[QuantScheme] = None) -> Tensor:
+        h = C.c_void_p()
+        c = scheme.to_c() if scheme is not None else None
+        check(lib().bq_pack_load(self.handle, name.encode(), C.byref(c) if c is not None else None, device.handle, C.byref(h)))
+        return _wrap(h, device)
+
+
+class PackWriter:
+    """burn-pack's `Writer`: tensors in the order added, 256-byte aligned, descriptors by name."""
+
+    def __init__(self):
+        h = C.c_void_p()
+        check(lib().bq_pack_writer_new(C.byref(h)))
+        self.handle = h
+
+    def __del__(self):
+        h, self.handle = getattr(self, "handle", None), None
+        if h:
+            lib().bq_pack_writer_free(h)
+
+    def with_metadata(self, key, value):
+        check(lib().bq_pack_writer_set_metadata(self.handle, key.encode(), value.encode()))
+        return self
+
+    def add_tensor(self, name, t: Tensor, param_id=None):
+        check(lib().bq_pack_writer_add_tensor(self.handle, name.encode(), t.handle, 0 if param_id is None else 1, param_id or 0))
+        return self
+
+    def add_bytes(self, name, dtype: str, shape, data: np.ndarray, scheme: Optional[QuantScheme] = None, param_id=None):
+        sh, rank = _shape_arg(shape)
+        buf = np.ascontiguousarray(data).view(np.uint8).reshape(-1)
+        c = scheme.to_c() if scheme is not None else None
+        check(lib().bq_pack_writer_add_bytes(self.handle, name.encode(), _lib.PACK_DTYPES.index(dtype), C.byref(c) if c is not None else None,
+                                             sh, rank, buf.ctypes.data if buf.size else None, buf.size,
+                                             0 if param_id is None else 1, param_id or 0))
+        return self
+
+    def size(self) -> int:
+        n = C.c_size_t()
+        check(lib().bq_pack_writer_size(self.handle, C.byref(n)))
+        return n.value
+
+    def into_bytes(self) -> np.ndarray:
+        out = np.empty(self.size(), np.uint8)
+        n = C.c_size_t()
+        check(lib().bq_pack_writer_write_into(self.handle, out.ctypes.data, out.size, C.byref(n)))
+        return out[: n.value]
+
+    def write_to_file(self, path):
+        check(lib().bq_pack_writer_write_file(self.handle, str(path).encode()))

@@ -226,6 +226,68 @@ bq_status bq_q_swap_dims(const bq_tensor* t, int32_t dim1, int32_t dim2, bq_tens
 bq_status bq_q_permute(const bq_tensor* t, const int32_t* axes, int32_t rank, bq_tensor** out);
 bq_status bq_q_flip(const bq_tensor* t, const int32_t* axes, int32_t n_axes, bq_tensor** out);
 
+/* ------------------------------------------------------------------ burnpack containers
+ * The on-disk format quantized modules are saved in (crates/burn-pack: base.rs:13-60 header and
+ * alignment, lib.rs:52-82 layout, writer.rs:257-314 offsets, reader.rs validation). A quantized
+ * tensor's bytes in the file are its QuantizedBytes blob (crates/burn-store/src/tensor_snapshot.rs:
+ * 253-262, crates/burn-pack/src/writer.rs:310-340), i.e. what bq_q_from_data takes: a tensor loads
+ * out of the mapped file with one host-to-device copy when its value bytes are a multiple of 256
+ * (two otherwise). DType tags follow the order of burn's DType enum
+ * (crates/burn-std/src/tensor/dtype.rs:10-26). */
+enum {
+  BQ_PACK_F64 = 0, BQ_PACK_F32, BQ_PACK_FLEX32, BQ_PACK_F16, BQ_PACK_BF16, BQ_PACK_I64, BQ_PACK_I32, BQ_PACK_I16,
+  BQ_PACK_I8, BQ_PACK_U64, BQ_PACK_U32, BQ_PACK_U16, BQ_PACK_U8, BQ_PACK_BOOL, BQ_PACK_QFLOAT
+};
+typedef struct bq_pack bq_pack;               /* an open container (Reader) */
+typedef struct bq_pack_writer bq_pack_writer; /* tensors collected for writing (Writer) */
+typedef struct bq_pack_entry {                /* one TensorDescriptor + where its bytes are */
+  const char* name;      /* owned by the bq_pack */
+  int32_t dtype;         /* BQ_PACK_* */
+  int32_t rank;
+  size_t shape[BQ_MAX_RANK];
+  uint64_t data_begin, data_end; /* data_offsets, relative to the data section */
+  int32_t has_param_id;
+  uint64_t param_id;
+  int32_t has_scheme;    /* QFloat whose scheme this library wrote and could read back */
+  bq_scheme scheme;
+  const uint8_t* data;   /* the tensor's bytes inside the mapped / borrowed container */
+} bq_pack_entry;
+/* aligned_data_section_start (base.rs:52-60): where the data section begins for a metadata size. */
+size_t bq_pack_data_section_start(size_t metadata_size);
+/* Reader::from_file / from_bytes. Only header and metadata are parsed; the file is memory-mapped
+ * and tensor bytes are touched when loaded. copy = 0 borrows `bytes` (must outlive the pack).
+ * Rejections follow the reader's: bad magic / version (BQ_ERR_DTYPE), a short header, oversized
+ * metadata, more tensors or bytes than the limits, a file smaller than its descriptors claim
+ * (BQ_ERR_SIZE). */
+bq_status bq_pack_open(const char* path, bq_pack** out);
+bq_status bq_pack_from_bytes(const uint8_t* bytes, size_t len, int32_t copy, bq_pack** out);
+bq_status bq_pack_close(bq_pack* pack);
+int64_t bq_pack_num_tensors(const bq_pack* pack);
+/* Entries in name order (the reference iterates a BTreeMap). */
+bq_status bq_pack_entry_at(const bq_pack* pack, int64_t index, bq_pack_entry* out);
+bq_status bq_pack_find(const bq_pack* pack, const char* name, bq_pack_entry* out);
+/* A user metadata value, or NULL. */
+const char* bq_pack_metadata(const bq_pack* pack, const char* key);
+/* The named tensor as a device tensor. QFloat entries take their scheme from `scheme`; NULL is
+ * accepted when the file was written by this library (how burn's own writer serializes a
+ * QuantScheme is decided outside the reference tree and is not relied on). F32 / BF16 entries load
+ * as float tensors; other dtypes are declined. */
+bq_status bq_pack_load(const bq_pack* pack, const char* name, const bq_scheme* scheme, bq_device* dev, bq_tensor** out);
+/* Writer: tensors are laid out in the order added, each at the next 256-byte boundary; descriptors
+ * are emitted in name order; a duplicate name or a byte length that cannot describe the declared
+ * dtype and shape is refused (writer.rs:264-330). add_tensor copies a device tensor back first. */
+bq_status bq_pack_writer_new(bq_pack_writer** out);
+bq_status bq_pack_writer_free(bq_pack_writer* w);
+bq_status bq_pack_writer_set_metadata(bq_pack_writer* w, const char* key, const char* value);
+bq_status bq_pack_writer_add_bytes(bq_pack_writer* w, const char* name, int32_t dtype, const bq_scheme* scheme,
+                                   const size_t* shape, int32_t rank, const uint8_t* data, size_t len,
+                                   int32_t has_param_id, uint64_t param_id);
+bq_status bq_pack_writer_add_tensor(bq_pack_writer* w, const char* name, const bq_tensor* t, int32_t has_param_id,
+                                    uint64_t param_id);
+bq_status bq_pack_writer_size(const bq_pack_writer* w, size_t* size_out);
+bq_status bq_pack_writer_write_into(const bq_pack_writer* w, uint8_t* buffer, size_t capacity, size_t* size_out);
+bq_status bq_pack_writer_write_file(const bq_pack_writer* w, const char* path);
+
 /* ------------------------------------------------------------------ kernel level
  * Plain pointers, no allocation. `stream` is a hipStream_t (NULL = the default stream).
  * A "run block" scheme is one whose blocks are `block` consecutive elements of the flat storage

@@ -656,6 +656,52 @@ def test_q_matmul_with_two_byte_scales(dev, sdt):
         matmul_check(out, ref)
 
 
+# ------------------------------------------------------------------ burnpack files
+
+def test_burnpack_round_trip_of_device_tensors(dev, tmp_path):
+    """Quantized and float tensors written to a .bpk file and loaded back into device memory:
+    every blob comes back byte for byte, straight out of the mapped file."""
+    from burn_amd import PackReader, PackWriter
+    rng = np.random.default_rng(90)
+    w = (rng.standard_normal((256, 512)) * 0.02).astype(np.float32)
+    cases = {
+        "layer.weight.q8_block": QuantScheme().per_block((32,)),
+        "layer.weight.q4_block": QuantScheme(value=QuantValue.Q4S).per_block((32,)),
+        "layer.weight.q8_tensor_native": QuantScheme(store=QuantStore.Native),
+        "layer.weight.q8_bf16_scales": QuantScheme().per_block((32,), ScaleDtype.BF16),
+        "layer.weight.ragged_native": QuantScheme(store=QuantStore.Native),      # value bytes not a multiple of 256
+    }
+    tensors, writer = {}, PackWriter().with_metadata("producer", "burn_amd tests")
+    for i, (name, scheme) in enumerate(cases.items()):
+        src = w[:3, :67] if "ragged" in name else w
+        tensors[name] = QTensorOps.quantize_dynamic(FloatOps.float_from_data(np.ascontiguousarray(src), dev), scheme)
+        writer.add_tensor(name, tensors[name], param_id=1000 + i)
+    bias = rng.standard_normal(512).astype(np.float32)
+    writer.add_tensor("layer.bias", FloatOps.float_from_data(bias, dev))
+    path = tmp_path / "model.bpk"
+    writer.write_to_file(path)
+    raw = path.read_bytes()
+    assert raw[:4] == b"NRUB" and len(raw) == writer.size()
+    reader = PackReader(tmp_path / "model")                     # the canonical extension is appended
+    assert len(reader) == len(cases) + 1 and reader.metadata("producer") == "burn_amd tests"
+    for i, (name, scheme) in enumerate(cases.items()):
+        e = reader.find(name)
+        blob = QTensorOps.q_into_data(tensors[name])
+        assert e["dtype"] == "QFloat" and e["scheme"] == scheme and e["param_id"] == 1000 + i
+        assert e["data_offsets"][0] % 256 == 0 and e["data_offsets"][1] - e["data_offsets"][0] == blob.bytes.size
+        for given in (None, scheme):                              # the file's own scheme, or the caller's
+            back = reader.load(name, dev, scheme=given)
+            assert back.shape == tensors[name].shape and back.scheme == scheme
+            assert QTensorOps.q_into_data(back).bytes.tobytes() == blob.bytes.tobytes()
+        d0 = FloatOps.float_into_data(QTensorOps.dequantize(tensors[name]))
+        d1 = FloatOps.float_into_data(QTensorOps.dequantize(reader.load(name, dev)))
+        assert d0.tobytes() == d1.tobytes()
+    assert FloatOps.float_into_data(reader.load("layer.bias", dev)).tobytes() == bias.tobytes()
+    # a scheme that does not describe the stored bytes is the reference's size mismatch
+    with pytest.raises(ba.BurnqError):
+        reader.load("layer.weight.q8_block", dev, scheme=QuantScheme(value=QuantValue.Q4S).per_block((32,)))
+
+
 # ------------------------------------------------------------------ the configs at full size
 
 def test_config1_per_tensor_q8s_native_4096(dev):

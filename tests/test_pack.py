@@ -1,0 +1,150 @@
+"""burnpack containers (crates/burn-pack): the format rules the reference's own tests hold --
+header constants and round trip (tests/header.rs), data-section alignment (tests/alignment.rs),
+reader rejections (tests/errors.rs) -- checked on the CPU against containers assembled by hand
+here, and the packed-Q4 byte lengths of crates/burn-store/src/tensor_snapshot.rs:517-541. The
+GPU round trip (device tensor -> file -> device tensor) is in test_gpu_parity.py."""
+import struct
+
+import numpy as np
+import pytest
+
+import burn_amd as ba
+from burn_amd import PackReader, PackWriter, QuantScheme, QuantStore, QuantValue, _lib
+
+
+# ---- a minimal CBOR encoder, independent of the library's (RFC 8949: shortest-form heads) -------
+def _head(major, v):
+    if v < 24:
+        return bytes([major << 5 | v])
+    for info, fmt, lim in ((24, ">B", 1 << 8), (25, ">H", 1 << 16), (26, ">I", 1 << 32), (27, ">Q", 1 << 64)):
+        if v < lim:
+            return bytes([major << 5 | info]) + struct.pack(fmt, v)
+    raise ValueError(v)
+
+
+def cbor(o):
+    if isinstance(o, bool):
+        return bytes([0xF5 if o else 0xF4])
+    if isinstance(o, int):
+        return _head(0, o)
+    if isinstance(o, str):
+        b = o.encode()
+        return _head(3, len(b)) + b
+    if isinstance(o, (list, tuple)):
+        return _head(4, len(o)) + b"".join(cbor(i) for i in o)
+    if isinstance(o, dict):
+        return _head(5, len(o)) + b"".join(cbor(k) + cbor(v) for k, v in o.items())
+    raise TypeError(type(o))
+
+
+def container(tensors, metadata=None, version=1, magic=0x4255524E):
+    """tensors: list of (name, dtype, shape, bytes) laid out in the given order, 256-byte aligned."""
+    desc, cur, chunks = {}, 0, []
+    for name, dtype, shape, data in tensors:
+        begin = (cur + 255) // 256 * 256
+        desc[name] = {"dtype": dtype, "shape": list(shape), "data_offsets": [begin, begin + len(data)]}
+        chunks.append((begin, data))
+        cur = begin + len(data)
+    meta = {"tensors": dict(sorted(desc.items()))}
+    if metadata:
+        meta["metadata"] = dict(sorted(metadata.items()))
+    m = cbor(meta)
+    start = (10 + len(m) + 255) // 256 * 256
+    out = bytearray(start + cur)
+    out[:10] = struct.pack("<IHI", magic, version, len(m))
+    out[10:10 + len(m)] = m
+    for begin, data in chunks:
+        out[start + begin:start + begin + len(data)] = data
+    return bytes(out)
+
+
+def test_header_constants_and_alignment():
+    """tests/header.rs `header_constants`, tests/alignment.rs `data_section_start_is_aligned`."""
+    assert struct.pack("<I", 0x4255524E) == b"NRUB"
+    L = _lib.lib()
+    for metadata_size in (0, 1, 10, 245, 246, 247, 4096):
+        start = L.bq_pack_data_section_start(metadata_size)
+        assert start % 256 == 0 and 10 + metadata_size <= start < 10 + metadata_size + 256
+    assert L.bq_pack_data_section_start(246) == 256 and L.bq_pack_data_section_start(247) == 512
+
+
+def test_reader_parses_a_hand_assembled_container():
+    a = np.float32([1, 2, 3]).tobytes()
+    b = np.float32([4]).tobytes()
+    raw = container([("b", "F32", (1,), b), ("a", "F32", (3,), a)], {"producer": "by hand"})
+    r = PackReader(raw)
+    assert len(r) == 2
+    ea, eb = r.entries()                              # name order, whatever the layout order
+    assert (ea["name"], ea["dtype"], ea["shape"]) == ("a", "F32", (3,))
+    assert eb["data_offsets"] == (0, 4) and ea["data_offsets"] == (256, 268)   # each tensor on a 256-byte boundary
+    assert r.metadata("producer") == "by hand" and r.metadata("missing") is None
+    import ctypes as C
+    assert C.string_at(ea["data_ptr"], 12) == a and C.string_at(eb["data_ptr"], 4) == b
+    with pytest.raises(ba.BurnqError, match="TensorNotFound"):
+        r.find("c")
+
+
+def test_reader_rejections():
+    """tests/header.rs / tests/errors.rs: bad magic, short input, unknown version, a container
+    smaller than its descriptors claim."""
+    good = container([("w", "F32", (2,), np.float32([1, 2]).tobytes())])
+    PackReader(good)
+    with pytest.raises(ba.BurnqError, match="InvalidMagicNumber"):
+        PackReader(container([("w", "F32", (2,), bytes(8))], magic=0xDEADBEEF))
+    with pytest.raises(ba.BurnqError, match="InvalidHeader"):
+        PackReader(bytes(4))
+    with pytest.raises(ba.BurnqError, match="InvalidVersion"):
+        PackReader(container([("w", "F32", (2,), bytes(8))], version=2))
+    with pytest.raises(ba.BurnqError, match="smaller than its tensors"):
+        PackReader(good[:-1])
+    with pytest.raises(ba.BurnqError, match="InvalidHeader"):
+        PackReader(good[:12])
+    with pytest.raises(ba.BurnqError, match="MetadataDeserializationError"):
+        PackReader(struct.pack("<IHI", 0x4255524E, 1, 3) + b"\xff\xff\xff" + bytes(300))
+
+
+def test_writer_emits_what_the_format_prescribes():
+    """The writer's bytes equal a container assembled by hand from the format rules: tensors laid
+    out in insertion order at 256-byte boundaries, descriptors and user metadata in key order,
+    shortest-form CBOR integers."""
+    a, b = np.float32([1, 2, 3]), np.float32([4])
+    w = PackWriter().with_metadata("producer", "test").add_bytes("b", "F32", (1,), b).add_bytes("a", "F32", (3,), a, param_id=42)
+    raw = w.into_bytes().tobytes()
+    desc_a = {"dtype": "F32", "shape": [3], "data_offsets": [256, 268], "param_id": 42}
+    desc_b = {"dtype": "F32", "shape": [1], "data_offsets": [0, 4]}
+    m = cbor({"tensors": {"a": desc_a, "b": desc_b}, "metadata": {"producer": "test"}})
+    assert raw[:10] == struct.pack("<IHI", 0x4255524E, 1, len(m)) and raw[10:10 + len(m)] == m
+    start = (10 + len(m) + 255) // 256 * 256
+    assert len(raw) == w.size() == start + 268
+    assert raw[10 + len(m):start] == bytes(start - 10 - len(m))          # zero padding
+    assert raw[start:start + 4] == b.tobytes() and raw[start + 256:start + 268] == a.tobytes()
+    # size / write_into agree (tests/alignment.rs), a buffer one byte short is refused
+    import ctypes as C
+    n = C.c_size_t()
+    small = np.empty(len(raw) - 1, np.uint8)
+    assert _lib.lib().bq_pack_writer_write_into(w.handle, small.ctypes.data, small.size, C.byref(n)) == _lib.ERR_SIZE
+    # duplicate names and impossible byte lengths are refused (writer.rs:264-330)
+    with pytest.raises(ba.BurnqError, match="Duplicate tensor name"):
+        w.add_bytes("a", "F32", (3,), a)
+    with pytest.raises(ba.BurnqError, match="TensorBytesSizeMismatch"):
+        PackWriter().add_bytes("x", "F32", (4,), a)
+
+
+def test_quantized_entries_carry_the_blob_length(kats):
+    """A QFloat tensor's bytes in the file are its QuantizedBytes blob; its length is
+    quantized_data_len (tensor_snapshot.rs:253-262). The packed-Q4 cases of tensor_snapshot.rs:517-541."""
+    scheme = QuantScheme(value=QuantValue.Q4S)
+    w = PackWriter()
+    for i, case in enumerate(kats["packed_q4_data_len"]["cases"]):
+        w.add_bytes(f"t{i}", "QFloat", case["shape"], np.zeros(case["len"], np.uint8), scheme=scheme)
+        with pytest.raises(ba.BurnqError, match="TensorBytesSizeMismatch"):
+            PackWriter().add_bytes("bad", "QFloat", case["shape"], np.zeros(case["len"] + 4, np.uint8), scheme=scheme)
+    r = PackReader(w.into_bytes())
+    for i, case in enumerate(kats["packed_q4_data_len"]["cases"]):
+        e = r.find(f"t{i}")
+        assert e["dtype"] == "QFloat" and e["data_offsets"][1] - e["data_offsets"][0] == case["len"]
+        assert e["data_offsets"][0] % 256 == 0 and e["scheme"] == scheme
+    # a block scheme with 2-byte scales survives the scheme round trip too
+    s2 = QuantScheme(store=QuantStore.Native).per_block((2, 16), ba.ScaleDtype.BF16)
+    w2 = PackWriter().add_bytes("q", "QFloat", (4, 32), np.zeros(4 * 32 + 2 * 4, np.uint8), scheme=s2)
+    assert PackReader(w2.into_bytes()).find("q")["scheme"] == s2
