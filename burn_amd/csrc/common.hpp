@@ -46,10 +46,13 @@ const char* get_error();
   } while (0)
 
 // ---- value helpers ---------------------------------------------------------------------------
-// QuantValue::range(): Q8S (-127,127), Q4S (-7,7).
+// QuantValue::range(): Q8S (-127,127), Q4S (-7,7), Q2S (-1,1) (ternary: -1, 0, +1).
+// value_known: what the fused kernels take. Q2S goes through the general kernels and the ternary
+// matmul only (value_supported).
 inline bool value_known(int v) { return v == BQ_Q8S || v == BQ_Q4S; }
-inline int value_bits(int v) { return v == BQ_Q8S ? 8 : 4; }
-inline int value_qmax(int v) { return v == BQ_Q8S ? 127 : 7; }
+inline bool value_supported(int v) { return value_known(v) || v == BQ_Q2S; }
+inline int value_bits(int v) { return v == BQ_Q8S ? 8 : (v == BQ_Q4S ? 4 : 2); }
+inline int value_qmax(int v) { return v == BQ_Q8S ? 127 : (v == BQ_Q4S ? 7 : 1); }
 inline int num_quants(int v) { return 32 / value_bits(v); }
 
 inline size_t round_up(size_t x, size_t a) { return (x + a - 1) / a * a; }
@@ -162,6 +165,12 @@ bq_status launch_qskinny(const void* x, int x_dtype, const uint32_t* w, const fl
 
 bool qgemm_ok(int a_dtype, size_t k, size_t n, int value, size_t scales_per_row);
 bool fused_matmul_ok(size_t m, size_t k, size_t n, int lhs_dtype, int value, size_t scales_per_row);
+
+// Per-tensor scale from the absmax cells of bqk_absmax_f32, rounded up to the scale dtype (quantize.hip).
+bq_status launch_scale_from_cells(const uint32_t* cells, int value, int scale_dtype, float* scale_out, hipStream_t stream);
+// Ternary matmul (qmatmul.hip): out[M,N] = gamma * sum_k t[k][n] * x[m][k] with t in {-1, 0, +1} packed 16 per word.
+bq_status launch_ternary_matmul(const float* x, const uint32_t* w, const float* scale, size_t m, size_t k, size_t n,
+                                float* out, hipStream_t stream);
 
 // dst[0..n) = value, as a kernel (safe to record into a HIP graph, unlike a memset node).
 bq_status launch_fill_u32(uint32_t* dst, size_t n, uint32_t value, hipStream_t stream);

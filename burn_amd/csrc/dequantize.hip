@@ -245,8 +245,10 @@ bq_status launch_dequantize_rect(const void* values, const size_t* shape, int ra
                      scales, out)
   if (value == BQ_Q8S) {
     if (bf16) BQ_RECT(8, true); else BQ_RECT(8, false);
-  } else {
+  } else if (value == BQ_Q4S) {
     if (bf16) BQ_RECT(4, true); else BQ_RECT(4, false);
+  } else {
+    if (bf16) BQ_RECT(2, true); else BQ_RECT(2, false);
   }
 #undef BQ_RECT
   BQ_HIP(hipGetLastError());

@@ -46,8 +46,8 @@ q_gather_kernel(const uint32_t* __restrict__ src, uint32_t* __restrict__ dst, si
     uint32_t v;
     if (BITS == 8)
       v = reinterpret_cast<const uint8_t*>(src)[idx];
-    else
-      v = (src[idx >> 3] >> (4 * (idx & 7))) & 0xFu;
+    else  // (rows are whole words, so flat element idx sits in word idx / EPW)
+      v = (src[idx / EPW] >> (BITS * (idx % EPW))) & ((1u << BITS) - 1u);
     word |= v << (BITS * j);
   }
   if (!native || e0 + EPW <= n) {
@@ -90,14 +90,17 @@ bq_status launch_q_gather(const void* src, void* dst, const size_t* src_shape, i
   for (int a = 0; a < rank; ++a) n *= src_shape[a];
   if (n == 0) return BQ_OK;
   const GatherDims d = make_dims(src_shape, rank, axes, flip);
-  const int epw = value == BQ_Q8S ? 4 : 8;
+  const int epw = num_quants(value);
   const size_t units = (n + epw - 1) / epw;
   dim3 grid(static_cast<unsigned>((units + 255) / 256)), tb(256);
   if (value == BQ_Q8S)
     hipLaunchKernelGGL(q_gather_kernel<8>, grid, tb, 0, st, static_cast<const uint32_t*>(src),
                        static_cast<uint32_t*>(dst), n, d, native);
-  else
+  else if (value == BQ_Q4S)
     hipLaunchKernelGGL(q_gather_kernel<4>, grid, tb, 0, st, static_cast<const uint32_t*>(src),
+                       static_cast<uint32_t*>(dst), n, d, false);
+  else
+    hipLaunchKernelGGL(q_gather_kernel<2>, grid, tb, 0, st, static_cast<const uint32_t*>(src),
                        static_cast<uint32_t*>(dst), n, d, false);
   BQ_HIP(hipGetLastError());
   return BQ_OK;

@@ -466,6 +466,57 @@ __global__ void bf16_to_f32_kernel(const uint16_t* __restrict__ src, size_t n, f
   if (i < n) dst[i] = bf16_to_f32(src[i]);
 }
 
+// Ternary weights (Q2S: -1, 0, +1, 16 per word) times f32 activations, without a multiply in the
+// sum: +1 adds the activation, -1 subtracts it, anything else leaves the sum alone, and the
+// per-tensor scale multiplies the finished sum once -- crates/burn-ndarray/src/ops/qtensor.rs:431-517.
+// A lane owns one packed word column (16 outputs) and RM activation rows and walks k in ascending
+// order, which is the reference's order of additions: the results are the reference's bit for bit.
+template <int RM>
+__global__ void __launch_bounds__(256)
+ternary_matmul_kernel(const float* __restrict__ x, const uint32_t* __restrict__ w, const float* __restrict__ scale,
+                      size_t M, size_t K, size_t NW, float* __restrict__ out) {
+  const size_t wc = static_cast<size_t>(blockIdx.x) * 256 + threadIdx.x;
+  const size_t m0 = static_cast<size_t>(blockIdx.y) * RM;
+  if (wc >= NW) return;
+  float acc[RM][16];
+#pragma unroll
+  for (int r = 0; r < RM; ++r)
+#pragma unroll
+    for (int j = 0; j < 16; ++j) acc[r][j] = 0.0f;
+  for (size_t k = 0; k < K; ++k) {
+    const uint32_t word = w[k * NW + wc];
+#pragma unroll
+    for (int r = 0; r < RM; ++r) {
+      const float xv = m0 + r < M ? x[(m0 + r) * K + k] : 0.0f;
+#pragma unroll
+      for (int j = 0; j < 16; ++j) {
+        const uint32_t f = (word >> (2 * j)) & 3u;  // two's complement: 1 = +1, 3 = -1, 0 and 2 are skipped
+        acc[r][j] = f == 1u ? acc[r][j] + xv : (f == 3u ? acc[r][j] - xv : acc[r][j]);
+      }
+    }
+  }
+  const float gamma = scale[0];
+  const size_t N = NW * 16;
+#pragma unroll
+  for (int r = 0; r < RM; ++r) {
+    if (m0 + r >= M) break;
+    vfloat4* dst = reinterpret_cast<vfloat4*>(out + (m0 + r) * N + wc * 16);
+#pragma unroll
+    for (int q = 0; q < 4; ++q)
+      dst[q] = vfloat4{acc[r][4 * q] * gamma, acc[r][4 * q + 1] * gamma, acc[r][4 * q + 2] * gamma, acc[r][4 * q + 3] * gamma};
+  }
+}
+
+bq_status launch_ternary_matmul(const float* x, const uint32_t* w, const float* scale, size_t m, size_t k, size_t n,
+                                float* out, hipStream_t st) {
+  if (m == 0 || n == 0) return BQ_OK;
+  const size_t nw = n / 16;
+  dim3 grid(static_cast<unsigned>((nw + 255) / 256), static_cast<unsigned>((m + 3) / 4)), tb(256);
+  hipLaunchKernelGGL(ternary_matmul_kernel<4>, grid, tb, 0, st, x, w, scale, m, k, nw, out);
+  BQ_HIP(hipGetLastError());
+  return BQ_OK;
+}
+
 bq_status launch_add_bias(void* out, int out_dtype, const float* bias, size_t m, size_t n, hipStream_t st) {
   if (m == 0 || n == 0) return BQ_OK;
   hipLaunchKernelGGL(add_bias_kernel, dim3(static_cast<unsigned>((m * n + 255) / 256)), dim3(256), 0, st, out,

@@ -359,7 +359,7 @@ __global__ void rect_quantize_kernel(const float* __restrict__ x, RectDims d, si
                                      size_t words_per_line, size_t total_words, bool native,
                                      const float* __restrict__ scales, uint32_t* __restrict__ out) {
   constexpr int NQ = 32 / BITS;
-  constexpr float QMAX = (BITS == 8) ? 127.0f : 7.0f;
+  constexpr float QMAX = (BITS == 8) ? 127.0f : (BITS == 4 ? 7.0f : 1.0f);
   constexpr uint32_t MASK = (1u << BITS) - 1u;
   size_t w = static_cast<size_t>(blockIdx.x) * blockDim.x + threadIdx.x;
   if (w >= total_words) return;
@@ -507,8 +507,11 @@ bq_status launch_quantize_rect(const float* x, const size_t* shape, int rank, co
   if (value == BQ_Q8S)
     hipLaunchKernelGGL(rect_quantize_kernel<8>, grid, tb, 0, st, x, d, last, wpl, total, native,
                        scales, static_cast<uint32_t*>(values));
-  else
+  else if (value == BQ_Q4S)
     hipLaunchKernelGGL(rect_quantize_kernel<4>, grid, tb, 0, st, x, d, last, wpl, total, native,
+                       scales, static_cast<uint32_t*>(values));
+  else
+    hipLaunchKernelGGL(rect_quantize_kernel<2>, grid, tb, 0, st, x, d, last, wpl, total, native,
                        scales, static_cast<uint32_t*>(values));
   BQ_HIP(hipGetLastError());
   return BQ_OK;
@@ -556,6 +559,13 @@ __global__ void scales_from_wire_kernel(const uint16_t* __restrict__ src, float*
   const size_t i = static_cast<size_t>(blockIdx.x) * blockDim.x + threadIdx.x;
   if (i >= n) return;
   dst[i] = sdt == 2 ? __uint_as_float(static_cast<uint32_t>(src[i]) << 16) : f16_bits_to_f32(src[i]);
+}
+
+bq_status launch_scale_from_cells(const uint32_t* cells, int value, int sdt, float* scale_out, hipStream_t st) {
+  hipLaunchKernelGGL(scale_from_cells_kernel, dim3(1), dim3(kThreads), 0, st, cells, 2.0f * static_cast<float>(value_qmax(value)),
+                     sdt, scale_out);
+  BQ_HIP(hipGetLastError());
+  return BQ_OK;
 }
 
 bq_status launch_round_scales(const float* src, float* dst, size_t n, int sdt, hipStream_t st) {

@@ -66,8 +66,8 @@ static size_t scale_size(const bq_scheme& s) { return s.scale_dtype == BQ_SCALE_
 // length formula alone (quantized_data_len) pads a ragged last dim to whole words instead.
 static bq_status check_scheme(const bq_scheme& s, const size_t* shape, int rank, bool storable = true) {
   if (rank < 1 || rank > BQ_MAX_RANK) BQ_FAIL(BQ_ERR_SHAPE, "rank %d outside 1..%d", rank, BQ_MAX_RANK);
-  if (!value_known(s.value))
-    BQ_FAIL(BQ_ERR_UNSUPPORTED_SCHEME, "Quantization not supported for value %d (Q8S and Q4S are)", s.value);
+  if (!value_supported(s.value))
+    BQ_FAIL(BQ_ERR_UNSUPPORTED_SCHEME, "Quantization not supported for value %d (Q8S, Q4S and Q2S are)", s.value);
   if (s.scale_dtype != BQ_SCALE_F32 && s.scale_dtype != BQ_SCALE_F16 && s.scale_dtype != BQ_SCALE_BF16)
     BQ_FAIL(BQ_ERR_UNSUPPORTED_SCHEME, "scale dtype %d is not supported (f32, f16 and bf16 are)", s.scale_dtype);
   if (s.level != BQ_LEVEL_TENSOR && s.level != BQ_LEVEL_BLOCK)
@@ -740,7 +740,21 @@ static bq_status quantize_impl(const bq_tensor* x, const bq_scheme* scheme, cons
     }
     if (n == 0) break;
     const long run = run_block(*scheme, x->shape, x->rank);
-    if (scheme->level == BQ_LEVEL_TENSOR) {
+    if (!value_known(scheme->value)) {
+      // Q2S: the general kernels (any block shape). Per tensor, the range comes from the absmax
+      // pass like every per-tensor quantize_dynamic.
+      const bool per_tensor = scheme->level == BQ_LEVEL_TENSOR;
+      if (per_tensor && dynamic) {
+        uint32_t* cells = reinterpret_cast<uint32_t*>(q->scales() + 1);
+        rc = bqk_absmax_f32(xin, n, cells, st);
+        if (rc == BQ_OK) rc = launch_scale_from_cells(cells, scheme->value, sdt, q->scales(), st);
+        if (rc != BQ_OK) break;
+      }
+      size_t blk[BQ_MAX_RANK];
+      block_dims(*scheme, x->rank, blk);
+      rc = launch_quantize_rect(xin, x->shape, x->rank, per_tensor ? nullptr : blk, scheme->value, scheme->store,
+                                dynamic && !per_tensor, sdt, q->data, q->scales(), st);
+    } else if (scheme->level == BQ_LEVEL_TENSOR) {
       if (dynamic) {
         // the absmax cells sit right behind the scale (the first pass writes every cell)
         uint32_t* cells = reinterpret_cast<uint32_t*>(q->scales() + 1);
@@ -791,14 +805,15 @@ extern "C" bq_status bq_dequantize(const bq_tensor* q, int32_t float_dtype, bq_t
   bq_status rc = BQ_OK;
   const long run = run_block(q->scheme, q->shape, q->rank);
   if (n == 0) {
-  } else if (run >= 0 && (run == 0 || (fused_block_ok(static_cast<int>(run), q->scheme.value) && run <= 512))) {
+  } else if (value_known(q->scheme.value) && run >= 0 &&
+             (run == 0 || (fused_block_ok(static_cast<int>(run), q->scheme.value) && run <= 512))) {
     rc = bqk_dequantize(q->data, n, static_cast<int32_t>(run), q->scales(), q->scheme.value,
                         q->scheme.store, float_dtype, f->data, st);
   } else {
     size_t blk[BQ_MAX_RANK];
     block_dims(q->scheme, q->rank, blk);
-    rc = launch_dequantize_rect(q->data, q->shape, q->rank, blk, q->scales(), q->scheme.value,
-                                q->scheme.store, float_dtype, f->data, st);
+    rc = launch_dequantize_rect(q->data, q->shape, q->rank, q->scheme.level == BQ_LEVEL_TENSOR ? nullptr : blk,
+                                q->scales(), q->scheme.value, q->scheme.store, float_dtype, f->data, st);
   }
   if (rc != BQ_OK) {
     bq_tensor_release(f);
@@ -905,8 +920,24 @@ static bq_status q_matmul_impl(const bq_tensor* lhs, const bq_tensor* rhs, int32
   hipStream_t st = dev->stream;
 
   // Fused path: float lhs x quantized rhs whose scales are per tensor or runs along N.
+  // Ternary fast path (crates/burn-ndarray/src/ops/qtensor.rs:442-517): f32 activations times a
+  // per-tensor Q2S 2-D weight, no bias, f32 out. Every other Q2S product dequantizes first.
+  if (!lq && rq && rhs->scheme.value == BQ_Q2S && rhs->scheme.level == BQ_LEVEL_TENSOR && lhs->dtype == BQ_F32 &&
+      out_dtype == BQ_F32 && rhs->rank == 2 && d.n % 16 == 0) {
+    bq_tensor* o = nullptr;
+    BQ_TRY(new_float(dev, BQ_F32, d.out_shape, d.rank, &o));
+    bq_status rc = launch_ternary_matmul(static_cast<const float*>(lhs->data), static_cast<const uint32_t*>(rhs->data),
+                                         rhs->scales(), d.m, d.k, d.n, static_cast<float*>(o->data), st);
+    if (rc == BQ_OK && bias != nullptr) rc = launch_add_bias(o->data, BQ_F32, bias, d.m, d.n, st);  // linear: matmul, then + bias
+    if (rc != BQ_OK) {
+      bq_tensor_release(o);
+      return rc;
+    }
+    *out = o;
+    return BQ_OK;
+  }
   long run = rq ? run_block(rhs->scheme, rhs->shape, rhs->rank) : -1;
-  bool fused = !lq && rq && run >= 0;
+  bool fused = !lq && rq && run >= 0 && value_known(rhs->scheme.value);
   if (fused && run > 0) {
     const size_t vpl = static_cast<size_t>(num_quants(rhs->scheme.value));
     const size_t bw = static_cast<size_t>(run) / vpl;

@@ -17,12 +17,13 @@ from . import _lib
 class QuantValue(IntEnum):
     Q8S = _lib.Q8S
     Q4S = _lib.Q4S
+    Q2S = _lib.Q2S   # ternary: -1, 0, +1
 
     def range(self) -> Tuple[float, float]:
-        return (-127.0, 127.0) if self == QuantValue.Q8S else (-7.0, 7.0)
+        return {QuantValue.Q8S: (-127.0, 127.0), QuantValue.Q4S: (-7.0, 7.0), QuantValue.Q2S: (-1.0, 1.0)}[self]
 
     def size_bits(self) -> int:
-        return 8 if self == QuantValue.Q8S else 4
+        return {QuantValue.Q8S: 8, QuantValue.Q4S: 4, QuantValue.Q2S: 2}[self]
 
 
 class QuantStore(IntEnum):

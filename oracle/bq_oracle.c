@@ -22,6 +22,7 @@ int bqo_value_range(int value, float* a, float* b) {
   switch (value) {
     case BQO_Q8S: *a = -127.0f; *b = 127.0f; return 0;
     case BQO_Q4S: *a = -7.0f; *b = 7.0f; return 0;
+    case BQO_Q2S: *a = -1.0f; *b = 1.0f; return 0;
     default: return -1;
   }
 }
@@ -31,6 +32,7 @@ int bqo_size_bits(int value) {
   switch (value) {
     case BQO_Q8S: return 8;
     case BQO_Q4S: return 4;
+    case BQO_Q2S: return 2;
     default: return -1;
   }
 }
@@ -538,5 +540,21 @@ void bqo_decode_scales(const uint8_t* in, size_t n, int dtype, float* out) {
       memcpy(&h, in + 2 * i, 2);
       out[i] = dtype == BQO_SCALE_F16 ? f32_from_f16(h) : bits_f32((uint32_t)h << 16);
     }
+  }
+}
+
+void bqo_ternary_matmul(const float* lhs, size_t m, size_t k, size_t n, const int8_t* rhs_q, float gamma, float* out) {
+  for (size_t i = 0; i < m; ++i) {
+    float* orow = out + i * n;
+    for (size_t j = 0; j < n; ++j) orow[j] = 0.0f;
+    for (size_t kk = 0; kk < k; ++kk) {
+      const float x = lhs[i * k + kk];
+      const int8_t* wrow = rhs_q + kk * n;
+      for (size_t j = 0; j < n; ++j) {
+        if (wrow[j] == 1) orow[j] += x;
+        else if (wrow[j] == -1) orow[j] -= x;
+      }
+    }
+    for (size_t j = 0; j < n; ++j) orow[j] *= gamma;
   }
 }

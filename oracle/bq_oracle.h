@@ -22,6 +22,13 @@
  *   bqo_encode/decode    burn-std/src/tensor/quantization.rs:605-625, tests .../quantization/data.rs:6-50
  *   bqo_block_of         ops/quantize.rs:171-206 + brute force against a reshape on small shapes
  *   bqo_q_matmul         ops/matmul.rs:141-168, :204-249 (known 3x4 and 3x16 products)
+ *   bqo_ternary_matmul   burn-ndarray/src/ops/qtensor.rs:431-517 restated loop for loop; its values are
+ *                        Q2S = {-1, 0, +1}: the range (-1, 1) is what that function's match arms and doc
+ *                        comment state (QuantValue::range() itself lives in cubecl-common, absent).
+ *                        Checked the way the reference checks it (ops/extended/ternary_matmul.rs, its
+ *                        inputs): equal to dequantize-then-matmul within f32 rounding, and exactly 0
+ *                        for an all-zero weight; the quantized ternary values of that test's weight
+ *                        follow from the same round / clamp rule the Q8S / Q4S vectors pin.
  *   bqo_scale_to_dtype   f32 / f16 / bf16. The rule is the reference's doc comment (burn-std
  *                        .../quantization.rs:354-368: "the smallest value representable by the scale
  *                        dtype that is no smaller"); its arithmetic lives in cubecl-common (absent).
@@ -47,7 +54,7 @@ extern "C" {
 
 #define BQO_MAX_RANK 8
 
-enum { BQO_Q8S = 0, BQO_Q4S = 1 };            /* QuantValue (symmetric signed ints only) */
+enum { BQO_Q8S = 0, BQO_Q4S = 1, BQO_Q2S = 2 }; /* QuantValue (symmetric signed ints only); Q2S = ternary */
 enum { BQO_LEVEL_TENSOR = 0, BQO_LEVEL_BLOCK = 1 };
 enum { BQO_STORE_NATIVE = 0, BQO_STORE_PACKED_U32 = 1 };
 enum { BQO_SCALE_F32 = 0, BQO_SCALE_F16 = 1, BQO_SCALE_BF16 = 2 };   /* ScaleDtype */
@@ -119,6 +126,10 @@ float bqo_scale_to_dtype(float scale, int dtype);
 size_t bqo_scale_size(int dtype);
 void bqo_encode_scales(const float* scales, size_t n, int dtype, uint8_t* out);
 void bqo_decode_scales(const uint8_t* in, size_t n, int dtype, float* out);
+
+/* ternary_matmul (burn-ndarray/src/ops/qtensor.rs:431-517): out[m][n] = gamma * sum over k, in
+ * ascending k, of +x (t = 1), -x (t = -1) or nothing (anything else); t = rhs_q[k][n]. */
+void bqo_ternary_matmul(const float* lhs, size_t m, size_t k, size_t n, const int8_t* rhs_q, float gamma, float* out);
 
 /* Threads used by the *_mt variants below (OpenMP), 1 when built without it. */
 int bqo_max_threads(void);

@@ -14,7 +14,7 @@ import numpy as np
 _HERE = os.path.dirname(os.path.abspath(__file__))
 _LIB_PATH = os.path.join(_HERE, "libbq_oracle.so")
 
-Q8S, Q4S = 0, 1
+Q8S, Q4S, Q2S = 0, 1, 2
 LEVEL_TENSOR, LEVEL_BLOCK = 0, 1
 STORE_NATIVE, STORE_PACKED_U32 = 0, 1
 MAX_RANK = 8
@@ -95,6 +95,8 @@ def lib():
         L.bqo_matmul_f32.restype = None
         L.bqo_q_matmul.argtypes = [pf, sz, pi8, psz, ps, pf, pf]
         L.bqo_max_threads.restype = i32
+        L.bqo_ternary_matmul.argtypes = [pf, sz, sz, sz, pi8, C.c_float, pf]
+        L.bqo_ternary_matmul.restype = None
         L.bqo_scale_to_dtype.argtypes = [C.c_float, i32]
         L.bqo_scale_to_dtype.restype = C.c_float
         L.bqo_scale_size.argtypes = [i32]
@@ -300,3 +302,13 @@ def encode_with_scale_dtype(q, scheme, scales, dtype):
     blob = encode(q, scheme, np.zeros_like(np.ascontiguousarray(scales, np.float32)))
     n = int(np.ascontiguousarray(scales).size)
     return np.concatenate([blob[: blob.size - 4 * n], encode_scales(scales, dtype)])
+
+
+def ternary_matmul(lhs, rhs_q, gamma):
+    lhs = np.ascontiguousarray(lhs, dtype=np.float32)
+    rhs_q = np.ascontiguousarray(rhs_q, dtype=np.int8)
+    m, k = lhs.shape
+    n = rhs_q.shape[1]
+    out = np.empty((m, n), np.float32)
+    lib().bqo_ternary_matmul(_p(lhs, C.c_float), m, k, n, _p(rhs_q, C.c_int8), float(gamma), _p(out, C.c_float))
+    return out

@@ -10,8 +10,8 @@ from __future__ import annotations
 
 import numpy as np
 
-RANGES = {"Q8S": (-127.0, 127.0), "Q4S": (-7.0, 7.0)}
-BITS = {"Q8S": 8, "Q4S": 4}
+RANGES = {"Q8S": (-127.0, 127.0), "Q4S": (-7.0, 7.0), "Q2S": (-1.0, 1.0)}
+BITS = {"Q8S": 8, "Q4S": 4, "Q2S": 2}
 
 
 def _block_dims(shape, block):
@@ -183,3 +183,14 @@ def scale_to_dtype(scales, dtype="F32"):
         r = np.where(np.isfinite(s), r, u)
         return r.astype(np.uint32).view(np.float32)
     raise ValueError(dtype)
+
+
+def ternary_matmul(lhs, q, gamma):
+    """crates/burn-ndarray/src/ops/qtensor.rs:431-517: +1 adds, -1 subtracts, anything else is
+    skipped, in ascending k; the per-tensor scale multiplies the finished sums."""
+    lhs = np.asarray(lhs, np.float32)
+    out = np.zeros((lhs.shape[0], q.shape[1]), np.float32)
+    for k in range(lhs.shape[1]):
+        x = lhs[:, k:k + 1]
+        out = np.where(q[k] == 1, out + x, np.where(q[k] == -1, out - x, out)).astype(np.float32)
+    return out * np.float32(gamma)

@@ -18,7 +18,7 @@ import burn_amd as ba  # noqa: E402
 from burn_amd import FloatOps, QTensorOps, QuantScheme, QuantStore, QuantValue, TensorData  # noqa: E402
 from burn_amd.quantization import ScaleDtype  # noqa: E402
 
-VAL = {QuantValue.Q8S: (co.Q8S, "Q8S"), QuantValue.Q4S: (co.Q4S, "Q4S")}
+VAL = {QuantValue.Q8S: (co.Q8S, "Q8S"), QuantValue.Q4S: (co.Q4S, "Q4S"), QuantValue.Q2S: (co.Q2S, "Q2S")}
 
 
 @pytest.fixture(scope="module")
@@ -654,6 +654,58 @@ def test_q_matmul_with_two_byte_scales(dev, sdt):
         out = FloatOps.float_into_data(QTensorOps.q_matmul(FloatOps.float_from_data(x, dev), tw))
         ref = no.q_matmul_f64(x, q_ref, s_ref, [32])
         matmul_check(out, ref)
+
+
+# ------------------------------------------------------------------ Q2S ternary weights
+
+@pytest.mark.parametrize("block", [None, (16,), (32,), (2, 32)])
+def test_q2s_quantize_dequantize(dev, block):
+    x = awkward((32, 96), 33)
+    scheme = QuantScheme(value=QuantValue.Q2S) if block is None else QuantScheme(value=QuantValue.Q2S).per_block(block)
+    tq, q_ref, s_ref, _ = check_quantize_dynamic(dev, x, scheme)
+    assert set(np.unique(q_ref).tolist()) <= {-1, 0, 1}
+    if block is None:   # layout ops carry 2-bit fields too
+        got, gs = unpack_blob(QTensorOps.q_into_data(QTensorOps.q_swap_dims(tq, 0, 1)))
+        assert (got == q_ref.T).all() and gs.reshape(-1).tobytes() == s_ref.reshape(-1).tobytes()
+
+
+def test_q2s_ternary_matmul_is_the_reference_sum(dev):
+    """f32 activations x per-tensor Q2S weight: the multiply-free path, bit for bit the reference's
+    loop (same order of additions), the reference test's own inputs first."""
+    a = np.float32([[0.5, -1.2, 0.3, 2.0], [1.0, 0.0, -0.7, 0.4], [-2.0, 1.5, 0.1, -0.3]])
+    w = np.zeros((4, 16), np.float32)
+    w[:, :3] = [[0.9, -0.2, 0.5], [-0.8, 0.1, 0.7], [0.0, 0.6, -0.4], [0.3, -0.9, 0.2]]   # padded to one packed word
+    scheme = QuantScheme(value=QuantValue.Q2S)
+    tw = QTensorOps.quantize_dynamic(FloatOps.float_from_data(w, dev), scheme)
+    q, s = unpack_blob(QTensorOps.q_into_data(tw))
+    assert q[:, :3].tolist() == [[1, 0, 1], [-1, 0, 1], [0, 1, 0], [0, -1, 0]] and s.reshape(-1)[0] == np.float32(0.9)
+    out = FloatOps.float_into_data(QTensorOps.q_matmul(FloatOps.float_from_data(a, dev), tw))
+    assert out.tobytes() == co.ternary_matmul(a, q, s.reshape(-1)[0]).tobytes()
+    ref = FloatOps.float_into_data(FloatOps.float_matmul(FloatOps.float_from_data(a, dev), QTensorOps.dequantize(tw)))
+    assert np.allclose(out, ref, rtol=2e-2, atol=1e-6)
+    # an all-zero weight: exactly 0
+    tz = QTensorOps.quantize_dynamic(FloatOps.float_from_data(np.zeros((3, 16), np.float32), dev), scheme)
+    z = FloatOps.float_into_data(QTensorOps.q_matmul(FloatOps.float_from_data(np.float32([[1.0, -2.0, 3.0]]), dev), tz))
+    assert (z == 0).all() and not np.isnan(z).any()
+    # larger shapes, ragged row counts, leading dims folded by linear, bias
+    from burn_amd import ModuleOps
+    rng = np.random.default_rng(58)
+    for m, k, n in ((1, 257, 64), (7, 512, 1040), (33, 96, 16)):
+        wr = rng.standard_normal((k, n)).astype(np.float32)
+        tw = QTensorOps.quantize_dynamic(FloatOps.float_from_data(wr, dev), scheme)
+        q, s = unpack_blob(QTensorOps.q_into_data(tw))
+        x = rng.standard_normal((m, k)).astype(np.float32)
+        got = FloatOps.float_into_data(QTensorOps.q_matmul(FloatOps.float_from_data(x, dev), tw))
+        assert got.tobytes() == co.ternary_matmul(x, q, s.reshape(-1)[0]).tobytes()
+        bias = rng.standard_normal(n).astype(np.float32)
+        lin = FloatOps.float_into_data(ModuleOps.linear(FloatOps.float_from_data(x.reshape(1, m, k), dev), tw,
+                                                        FloatOps.float_from_data(bias, dev)))
+        assert lin.shape == (1, m, n) and lin.reshape(m, n).tobytes() == (got + bias).astype(np.float32).tobytes()
+    # per-block Q2S and bf16 activations take the dequantize route, like the reference
+    twb = QTensorOps.quantize_dynamic(FloatOps.float_from_data(wr, dev), QuantScheme(value=QuantValue.Q2S).per_block((16,)))
+    qb, sb = unpack_blob(QTensorOps.q_into_data(twb))
+    gotb = FloatOps.float_into_data(QTensorOps.q_matmul(FloatOps.float_from_data(x, dev), twb))
+    matmul_check(gotb, no.q_matmul_f64(x, qb, sb, [16]))
 
 
 # ------------------------------------------------------------------ burnpack files

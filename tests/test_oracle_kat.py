@@ -382,3 +382,34 @@ def test_scale_to_dtype_survives_the_codec_like_the_reference_test():
     # exactly representable values pin the byte layout (as in the reference's two-level layout test)
     assert co.encode_scales(np.float32([0.5, 0.125]), co.SCALE_F16).view(np.uint16).tolist() == [0x3800, 0x3000]
     assert co.encode_scales(np.float32([0.5, 0.125]), co.SCALE_BF16).view(np.uint16).tolist() == [0x3F00, 0x3E00]
+
+
+# ------------------------------------------------------------------ Q2S ternary values
+
+def test_ternary_matmul_as_the_reference_checks_it():
+    """crates/burn-backend-tests/tests/tensor/float/quantization/ops/extended/ternary_matmul.rs with
+    its inputs: the multiply-free product equals dequantize-then-matmul (relative 2e-2 there), an
+    all-zero weight gives exactly 0. The ternary values of its weight follow from the round / clamp
+    rule with the range (-1, 1); C and numpy restatements agree bit for bit."""
+    a = np.float32([[0.5, -1.2, 0.3, 2.0], [1.0, 0.0, -0.7, 0.4], [-2.0, 1.5, 0.1, -0.3]])
+    w = np.float32([[0.9, -0.2, 0.5], [-0.8, 0.1, 0.7], [0.0, 0.6, -0.4], [0.3, -0.9, 0.2]])
+    sch = co.Scheme.make(co.Q2S, None, co.STORE_NATIVE)
+    q, s = co.quantize_dynamic(w, sch)
+    assert s.reshape(-1)[0] == np.float32(0.9)                      # (2 * 0.9) / (1 - (-1))
+    assert q.tolist() == [[1, 0, 1], [-1, 0, 1], [0, 1, 0], [0, -1, 0]]
+    qn, sn = no.quantize_dynamic(w, "Q2S")
+    assert (qn == q).all() and sn.reshape(-1)[0] == s.reshape(-1)[0]
+    native = co.ternary_matmul(a, q, s.reshape(-1)[0])
+    assert native.tobytes() == no.ternary_matmul(a, q, s.reshape(-1)[0]).tobytes()
+    reference = a.astype(np.float64) @ co.dequantize(q, sch, s).astype(np.float64)
+    assert np.allclose(native, reference, rtol=2e-2, atol=0)
+    # by hand, first row: 0.9 * (0.5 + 1.2) = 1.53, 0.9 * (0.3 - 2.0) = -1.53, 0.9 * (0.5 - 1.2) = -0.63
+    assert np.allclose(native[0], [1.53, -1.53, -0.63], rtol=1e-6)
+    zero = np.zeros((3, 1), np.float32)
+    qz, sz = co.quantize_dynamic(zero, sch)
+    assert (co.ternary_matmul(np.float32([[1.0, -2.0, 3.0]]), qz, sz.reshape(-1)[0]) == 0).all()
+    # packing: 16 values per word, low field first, two's complement fields
+    vals = np.int8([1, -1, 0, 1] * 4).reshape(1, 16)
+    word = co.pack_u32(vals, co.Q2S)
+    assert word.reshape(-1)[0] == sum(((v & 3) << (2 * i)) for i, v in enumerate([1, -1, 0, 1] * 4))
+    assert (co.unpack_u32(word, (1, 16), co.Q2S) == vals).all()
