@@ -16,6 +16,8 @@
 //     f32 accumulation.
 #include <algorithm>
 
+#include <type_traits>
+
 #include "common.hpp"
 #include "device_math.hpp"
 
@@ -201,53 +203,74 @@ qgemv1_kernel(const void* __restrict__ x, const uint32_t* __restrict__ w,
       s = 0.0f;
     }
   };
+  // An infinity or a NaN among this workgroup's activations (rows_per_wg x M of them, read once
+  // here, ahead of the weight loads) sends the whole workgroup through the guarded copy of the
+  // loop: xs * u - BIAS * xs would be inf - inf there, and a padded row's x[k_begin] * 0 would be
+  // NaN. Finite slices run the plain copy and pay one small load and a barrier for the test.
+  int bad = 0;
+  {
+    const size_t rows = k_end > k_begin ? k_end - k_begin : 0;
+    for (size_t i = threadIdx.x; i < rows * M; i += static_cast<size_t>(WAVES) * kWave) {
+      const size_t e = (i / rows) * K + k_begin + i % rows;
+      const uint32_t bits = X_BF16 ? static_cast<uint32_t>(static_cast<const uint16_t*>(x)[e]) << 16
+                                   : static_cast<const uint32_t*>(x)[e];
+      bad |= (bits & 0x7F800000u) == 0x7F800000u;
+    }
+  }
   LoadT q[U], qn[U];
   float sc[U], sn[U];
   size_t kb = k_begin + static_cast<size_t>(wave);
 #pragma unroll
   for (int u = 0; u < U; ++u) fetch(kb + static_cast<size_t>(u) * WAVES, q[u], sc[u]);
-  while (kb < k_end) {
-    const size_t kn = kb + static_cast<size_t>(WAVES) * U;
+  const bool nonfinite = __syncthreads_or(bad) != 0;
+  auto run = [&](auto G) {
+    constexpr bool guard = decltype(G)::value;
+    while (kb < k_end) {
+      const size_t kn = kb + static_cast<size_t>(WAVES) * U;
 #pragma unroll
-    for (int u = 0; u < U; ++u) fetch(kn + static_cast<size_t>(u) * WAVES, qn[u], sn[u]);
-    __builtin_amdgcn_sched_barrier(0);
+      for (int u = 0; u < U; ++u) fetch(kn + static_cast<size_t>(u) * WAVES, qn[u], sn[u]);
+      __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-    for (int u = 0; u < U; ++u) {
-      const size_t k = kb + static_cast<size_t>(u) * WAVES;
-      const size_t kx = k < k_end ? k : k_begin;  // rows past the slice: s is 0 there
-      const float sv = (PER_TENSOR || !(active && k < k_end)) ? sc[u] : valid_scale(sc[u]);
-      float xs[M];
+      for (int u = 0; u < U; ++u) {
+        const size_t k = kb + static_cast<size_t>(u) * WAVES;
+        const size_t kx = k < k_end ? k : k_begin;  // rows past the slice: s is 0 there
+        const float sv = (PER_TENSOR || !(active && k < k_end)) ? sc[u] : valid_scale(sc[u]);
+        float xs[M];
 #pragma unroll
-      for (int m = 0; m < M; ++m) {
-        const size_t e = static_cast<size_t>(m) * K + kx;
-        float xe;
-        if (X_BF16) {
-          const uint32_t pair = static_cast<const uint32_t*>(x)[e >> 1];
-          xe = __builtin_bit_cast(float, (e & 1) ? (pair & 0xFFFF0000u) : (pair << 16));
-        } else {
-          xe = static_cast<const float*>(x)[e];
+        for (int m = 0; m < M; ++m) {
+          const size_t e = static_cast<size_t>(m) * K + kx;
+          float xe;
+          if (X_BF16) {
+            const uint32_t pair = static_cast<const uint32_t*>(x)[e >> 1];
+            xe = __builtin_bit_cast(float, (e & 1) ? (pair & 0xFFFF0000u) : (pair << 16));
+          } else {
+            xe = static_cast<const float*>(x)[e];
+          }
+          if (guard) xe = k < k_end ? xe : 0.0f;
+          xs[m] = xe * sv;
+          if (!guard) corr[m] += xs[m];
         }
-        xs[m] = xe * sv;
-        corr[m] += xs[m];
+#pragma unroll
+        for (int i = 0; i < WPL; ++i) {
+          float f[VPL];
+          gemv1_fields<VPL>(q[u][i], f);
+#pragma unroll
+          for (int m = 0; m < M; ++m)
+#pragma unroll
+            for (int j = 0; j < VPL; ++j)
+              acc[m][i * VPL + j] = __builtin_fmaf(xs[m], guard ? f[j] - BIAS : f[j], acc[m][i * VPL + j]);
+        }
       }
+      __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-      for (int i = 0; i < WPL; ++i) {
-        float f[VPL];
-        gemv1_fields<VPL>(q[u][i], f);
-#pragma unroll
-        for (int m = 0; m < M; ++m)
-#pragma unroll
-          for (int j = 0; j < VPL; ++j) acc[m][i * VPL + j] = __builtin_fmaf(xs[m], f[j], acc[m][i * VPL + j]);
+      for (int u = 0; u < U; ++u) {
+        q[u] = qn[u];
+        sc[u] = sn[u];
       }
+      kb = kn;
     }
-    __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-    for (int u = 0; u < U; ++u) {
-      q[u] = qn[u];
-      sc[u] = sn[u];
-    }
-    kb = kn;
-  }
+  };
+  if (!nonfinite) run(std::false_type{}); else run(std::true_type{});
   // Sum the waves in a fixed order through LDS, one activation row at a time. Every wave stores
   // its CPL x 64 partials; then each thread adds up, over the waves, the outputs t, t + THREADS,
   // ... of the workgroup's CPL * 64 consecutive columns, so the stores to `part` are contiguous.

@@ -32,6 +32,7 @@
 // two halves are added through LDS, the K slices by qgemv_reduce_kernel, both in a fixed order
 // (no float atomics).
 #include <algorithm>
+#include <type_traits>
 
 #include "common.hpp"
 #include "device_math.hpp"
@@ -195,14 +196,28 @@ qsplit_kernel(const void* __restrict__ x, const uint32_t* __restrict__ w, const 
       }
     }
   };
-  auto split = [&](const float* t, uint32_t* hi, uint32_t* lo) {
+  // G (a std::bool_constant): the guarded variant, taken only by workgroups whose activation slice
+  // holds an infinity or a NaN. There the second term of a non-finite product is dropped (inf - inf
+  // would make every output of the row NaN, where the reference's sum has +-inf, and NaN only
+  // against a zero weight), Q4S weights are converted to their true values instead of the offset
+  // patterns (inf * (q + 136) - inf * 136 is NaN), and the padded step past the end is skipped
+  // (inf * 0). Finite slices never execute any of it.
+  auto split = [&](auto G, const float* t, uint32_t* hi, uint32_t* lo) {
+    constexpr bool guard = decltype(G)::value;
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
       hi[i] = pack_bf16(t[2 * i], t[2 * i + 1]);
-      lo[i] = pack_bf16(t[2 * i] - as_float(hi[i] << 16), t[2 * i + 1] - as_float(hi[i] & 0xFFFF0000u));
+      const float h0 = as_float(hi[i] << 16), h1 = as_float(hi[i] & 0xFFFF0000u);
+      float d0 = t[2 * i] - h0, d1 = t[2 * i + 1] - h1;
+      if (guard) {
+        d0 = (as_bits(h0) & 0x7F800000u) == 0x7F800000u ? 0.0f : d0;
+        d1 = (as_bits(h1) & 0x7F800000u) == 0x7F800000u ? 0.0f : d1;
+      }
+      lo[i] = pack_bf16(d0, d1);
     }
   };
-  auto multiply = [&](int buf, int s) {
+  auto multiply = [&](auto G, int buf, int s) {
+    constexpr bool guard = decltype(G)::value;
     const int sx = s < steps ? s : 0;  // past the end the weights are zeros: any finite activations do
     const uint32_t kl = static_cast<uint32_t>(h) * k_per_way + static_cast<uint32_t>(sx) * kStepRows + 8u * kg;
     float xv[MT][8];
@@ -229,7 +244,7 @@ qsplit_kernel(const void* __restrict__ x, const uint32_t* __restrict__ w, const 
       float v[8];
 #pragma unroll
       for (int r = 0; r < 8; ++r) v[r] = xv[0][r] * sr[r];
-      split(v, hi[0], lo[0]);
+      split(G, v, hi[0], lo[0]);
     }
     if (PER_TENSOR) {
 #pragma unroll
@@ -237,7 +252,7 @@ qsplit_kernel(const void* __restrict__ x, const uint32_t* __restrict__ w, const 
         float v[8];
 #pragma unroll
         for (int r = 0; r < 8; ++r) v[r] = xv[t][r] * (s < steps ? s_tensor : 0.0f);
-        split(v, hi[t], lo[t]);
+        split(G, v, hi[t], lo[t]);
       }
     }
 #pragma unroll
@@ -251,7 +266,7 @@ qsplit_kernel(const void* __restrict__ x, const uint32_t* __restrict__ w, const 
           float v[8];
 #pragma unroll
           for (int r = 0; r < 8; ++r) v[r] = xv[t][r] * sr[r];
-          split(v, hi[t], lo[t]);
+          split(G, v, hi[t], lo[t]);
         }
       }
       uint32_t b0[4], b1[4];
@@ -261,6 +276,12 @@ qsplit_kernel(const void* __restrict__ x, const uint32_t* __restrict__ w, const 
           const uint32_t p = __builtin_amdgcn_perm(wq[u][2 * i + 1], wq[u][2 * i], sel);
           b0[i] = __builtin_amdgcn_perm(as_bits(byte_to_float(p, 1)), as_bits(byte_to_float(p, 0)), 0x07060302u);
           b1[i] = __builtin_amdgcn_perm(as_bits(byte_to_float(p, 3)), as_bits(byte_to_float(p, 2)), 0x07060302u);
+        } else if (guard) {
+          // the nibbles' own values (q = (n ^ 8) - 8, exact in bf16: the upper half of the f32)
+          const uint32_t na = (wq[u][2 * i] >> nib_shift) & 0x000F000Fu, nb = (wq[u][2 * i + 1] >> nib_shift) & 0x000F000Fu;
+          auto qf = [](uint32_t n) { return as_bits(static_cast<float>(static_cast<int>(n ^ 8u) - 8)); };
+          b0[i] = __builtin_amdgcn_perm(qf(nb & 0xFu), qf(na & 0xFu), 0x07060302u);
+          b1[i] = __builtin_amdgcn_perm(qf(nb >> 16), qf(na >> 16), 0x07060302u);
         } else {
           // nibble n (two's complement) -> bf16 bits 0x4300 | (n ^ 8) = 128 + (q + 8) = q + 136, both
           // nibbles of the lane at once; the 136 is taken out again by the constant operand below
@@ -280,13 +301,13 @@ qsplit_kernel(const void* __restrict__ x, const uint32_t* __restrict__ w, const 
         const bf16x8 a_lo = __builtin_bit_cast(bf16x8, vuint4{lo[t][0], lo[t][1], lo[t][2], lo[t][3]});
         acc[t][u][0] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a_hi, bq0, acc[t][u][0], 0, 0, 0);
         acc[t][u][1] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a_hi, bq1, acc[t][u][1], 0, 0, 0);
-        if (VPL == 8) {
+        if (VPL == 8 && !guard) {
           acc[t][u][0] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a_hi, minus, acc[t][u][0], 0, 0, 0);
           acc[t][u][1] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a_hi, minus, acc[t][u][1], 0, 0, 0);
         }
         acc[t][u][0] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a_lo, bq0, acc[t][u][0], 0, 0, 0);
         acc[t][u][1] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a_lo, bq1, acc[t][u][1], 0, 0, 0);
-        if (VPL == 8) {
+        if (VPL == 8 && !guard) {
           acc[t][u][0] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a_lo, minus, acc[t][u][0], 0, 0, 0);
           acc[t][u][1] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a_lo, minus, acc[t][u][1], 0, 0, 0);
         }
@@ -297,6 +318,7 @@ qsplit_kernel(const void* __restrict__ x, const uint32_t* __restrict__ w, const 
   // The activation loads go first: loads return in order, and the first multiply needs the
   // activations and the first step of weights only, not everything that is in flight behind them.
   // (Buffer loads: rows past M and columns past K read as zero through the range check.)
+  int bad = 0;
   {
     constexpr uint32_t XB = X_BF16 ? 2u : 4u;  // bytes per activation
     const __amdgpu_buffer_rsrc_t rsrc_x =
@@ -325,19 +347,34 @@ qsplit_kernel(const void* __restrict__ x, const uint32_t* __restrict__ w, const 
       const uint32_t idx = static_cast<uint32_t>(tid) + static_cast<uint32_t>(i) * kSplitThreads;
       const uint32_t m = idx / vecs_per_row, kk = (idx % vecs_per_row) * 4u;
       if (idx < total) *reinterpret_cast<vuint4*>(xs + m * xpitch + kk) = v[i];
+      // an exponent field of all ones: an infinity or a NaN among this thread's activations
+      const uint32_t e = 0x7F800000u;
+      bad |= (v[i].x & e) == e || (v[i].y & e) == e || (v[i].z & e) == e || (v[i].w & e) == e;
     }
   }
-  __syncthreads();
+  const bool nonfinite = __syncthreads_or(bad) != 0;
 
   // (scheduling barriers: left alone, the compiler sinks a step's loads below the other step's
   // MFMAs to save registers, which puts the load latency in series with the arithmetic)
-  for (int s0 = 0; s0 < steps; s0 += kDepth) {
+  if (!nonfinite) {
+    for (int s0 = 0; s0 < steps; s0 += kDepth) {
 #pragma unroll
-    for (int b = 0; b < kDepth; ++b) {
-      multiply(b, s0 + b);
-      __builtin_amdgcn_sched_barrier(0);
-      fetch(b, s0 + b + kDepth);
-      __builtin_amdgcn_sched_barrier(0);
+      for (int b = 0; b < kDepth; ++b) {
+        multiply(std::false_type{}, b, s0 + b);
+        __builtin_amdgcn_sched_barrier(0);
+        fetch(b, s0 + b + kDepth);
+        __builtin_amdgcn_sched_barrier(0);
+      }
+    }
+  } else {
+    for (int s0 = 0; s0 < steps; s0 += kDepth) {
+#pragma unroll
+      for (int b = 0; b < kDepth; ++b) {
+        if (s0 + b < steps) multiply(std::true_type{}, b, s0 + b);
+        __builtin_amdgcn_sched_barrier(0);
+        fetch(b, s0 + b + kDepth);
+        __builtin_amdgcn_sched_barrier(0);
+      }
     }
   }
 

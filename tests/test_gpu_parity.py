@@ -937,6 +937,53 @@ def test_q_matmul_small_batches(dev, value, block, m, k, n):
 
 
 @pytest.mark.parametrize("value", [QuantValue.Q8S, QuantValue.Q4S])
+@pytest.mark.parametrize("block", [None, (32,), (64,)])
+@pytest.mark.parametrize("m,k,n", [(1, 4096, 1024), (1, 100, 64), (2, 96, 256), (4, 1056, 640), (8, 96, 128),
+                                   (8, 4096, 512), (16, 2080, 1152), (24, 96, 128), (64, 1024, 512),
+                                   (130, 264, 256)])
+def test_q_matmul_infinite_and_nan_activations(dev, value, block, m, k, n):
+    """The reference multiplies by the dequantized weights: an infinite activation gives +-inf in
+    its row (NaN where the weight is zero or where both signs meet), a NaN activation a NaN row,
+    and every other row stays finite. The kernels' shortcuts (offset weight fields, activations
+    split into two bf16 terms, zero-filled padding) must not turn that into something else."""
+    if block and n % block[0]:
+        pytest.skip("block does not divide N")
+    rng = np.random.default_rng(m * 31 + k + n)
+    w = (rng.standard_normal((k, n)) * 0.05).astype(np.float32)
+    w[rng.random((k, n)) < 0.05] = 0.0            # zero weights: inf * 0 = NaN
+    x = rng.standard_normal((m, k)).astype(np.float32)
+    x[0, 5 % k] = np.inf                           # (row 0 of a slice: the row that padding re-reads)
+    if m >= 2:
+        x[m - 1, k - 1] = -np.inf
+    if m >= 4:
+        x[2, k // 2] = np.inf
+        x[2, k // 3] = -np.inf                     # both signs in one row: NaN everywhere
+        x[3, k // 5] = np.nan
+    scheme = QuantScheme(value=value, block=block)
+    tq = QTensorOps.quantize_dynamic(FloatOps.float_from_data(w, dev), scheme)
+    q, s = unpack_blob(QTensorOps.q_into_data(tq))
+    with np.errstate(invalid="ignore", over="ignore"):
+        ref = no.q_matmul_f64(x, q, s, list(block) if block else None)
+
+    def same(out, ref):
+        assert (np.isnan(out) == np.isnan(ref)).all(), (np.isnan(out).sum(), np.isnan(ref).sum())
+        inf = np.isinf(ref)
+        assert (np.isinf(out) == inf).all()
+        assert (np.sign(out[inf]) == np.sign(ref[inf])).all()
+        fin = np.isfinite(ref)
+        assert fin.any() or m <= 2
+        if fin.any():
+            assert np.abs(out[fin] - ref[fin]).max() <= 1e-2 * np.abs(ref[fin]).max() + 1e-2
+
+    same(FloatOps.float_into_data(QTensorOps.q_matmul(FloatOps.float_from_data(x, dev), tq)), ref)
+    xb = ba.bf16_bits_from_f32(x)
+    with np.errstate(invalid="ignore", over="ignore"):
+        refb = no.q_matmul_f64(ba.f32_from_bf16_bits(xb), q, s, list(block) if block else None)
+    same(FloatOps.float_into_data(
+        QTensorOps.q_matmul(FloatOps.float_from_data(xb, dev, ba.BF16), tq, out_dtype=ba.F32)), refb)
+
+
+@pytest.mark.parametrize("value", [QuantValue.Q8S, QuantValue.Q4S])
 @pytest.mark.parametrize("block", [None, (32,)])
 @pytest.mark.parametrize("m,k,n", [(64, 1024, 512), (200, 2112, 768), (40, 4096, 1024), (129, 520, 256)])
 def test_q_matmul_split_k_tiles(dev, value, block, m, k, n):
