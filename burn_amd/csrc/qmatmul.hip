@@ -408,60 +408,91 @@ bool gemv1_ok(size_t m, size_t n, int lhs_dtype, int block, int value) {
 }
 
 // ================================================================================ float GEMM
-// Plain tiled f32 GEMM for the combinations where no operand stays quantized (quantized lhs x
-// float rhs, two quantized operands, rectangle blocks): both are dequantized first, as the
-// reference does. 64x64 tile, 16-deep, 4x4 outputs per thread. Not a tuned path.
+// f32-accurate GEMM on the matrix cores (v_mfma_f32_32x32x2_f32: full f32 products and sums) for the
+// combinations where no operand stays packed: quantized lhs x float rhs, rectangle blocks, ternary
+// weights outside the fast path. Both operands are dequantized first, as the reference does. A
+// workgroup of 4 waves (2 x 2) owns a (64 * WT)^2 tile, 16 deep; the next slab is loaded into
+// registers while the current one is multiplied out of LDS. Any shape, f32 or bf16 operands,
+// element-wise guarded loads: sized for correctness at a fair speed, not tuned to the limit.
 __device__ __forceinline__ float load_elem(const void* p, int dtype, size_t i) {
   return dtype == BQ_BF16 ? bf16_to_f32(static_cast<const uint16_t*>(p)[i])
                           : static_cast<const float*>(p)[i];
 }
 
+template <int WT>
 __global__ void __launch_bounds__(256)
 float_matmul_kernel(const void* __restrict__ a, int a_dtype, const void* __restrict__ b,
                     int b_dtype, size_t M, size_t K, size_t N, int out_dtype,
                     void* __restrict__ out) {
-  constexpr int T = 64, TK = 16;
-  __shared__ float As[TK][T + 1];
-  __shared__ float Bs[TK][T + 1];
-  const int tx = threadIdx.x % 16, ty = threadIdx.x / 16;
+  constexpr int T = 64 * WT, TK = 16, LD = T + 4, PER = T * TK / 256;
+  typedef float vfloat16 __attribute__((ext_vector_type(16)));
+  __shared__ float As[TK][LD];  // [k][row]: a wave's 32 rows of one k are consecutive words
+  __shared__ float Bs[TK][LD];  // [k][column]
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int wm = wave >> 1, wn = wave & 1;
   const size_t m0 = static_cast<size_t>(blockIdx.y) * T, n0 = static_cast<size_t>(blockIdx.x) * T;
-  float acc[4][4] = {};
+  vfloat16 acc[WT][WT];
+#pragma unroll
+  for (int i = 0; i < WT; ++i)
+#pragma unroll
+    for (int j = 0; j < WT; ++j)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.0f;
+
+  float ra[PER], rb[PER];
+  auto gload = [&](size_t kt) {
+#pragma unroll
+    for (int i = 0; i < PER; ++i) {
+      const int idx = tid + i * 256;
+      const size_t gr = m0 + idx / TK, gk = kt + idx % TK;   // A: k fastest, as in memory
+      ra[i] = (gr < M && gk < K) ? load_elem(a, a_dtype, gr * K + gk) : 0.0f;
+      const size_t gk2 = kt + idx / T, gn = n0 + idx % T;    // B: column fastest
+      rb[i] = (gk2 < K && gn < N) ? load_elem(b, b_dtype, gk2 * N + gn) : 0.0f;
+    }
+  };
+  gload(0);
   for (size_t kt = 0; kt < K; kt += TK) {
-    for (int i = threadIdx.x; i < T * TK; i += 256) {
-      int r = i / TK, c = i % TK;  // A: row r of tile, k c
-      size_t gr = m0 + r, gk = kt + c;
-      As[c][r] = (gr < M && gk < K) ? load_elem(a, a_dtype, gr * K + gk) : 0.0f;
-      int kr = i / T, nc = i % T;  // B: k kr, col nc
-      size_t gk2 = kt + kr, gn = n0 + nc;
-      Bs[kr][nc] = (gk2 < K && gn < N) ? load_elem(b, b_dtype, gk2 * N + gn) : 0.0f;
+#pragma unroll
+    for (int i = 0; i < PER; ++i) {
+      const int idx = tid + i * 256;
+      As[idx % TK][idx / TK] = ra[i];
+      Bs[idx / T][idx % T] = rb[i];
     }
     __syncthreads();
+    if (kt + TK < K) gload(kt + TK);
 #pragma unroll
-    for (int k = 0; k < TK; ++k) {
-      float av[4], bv[4];
+    for (int kk = 0; kk < TK; kk += 2) {
+      // operands of one 32x32x2 step: lane l holds A[row l % 32][k l / 32] and B[k l / 32][column l % 32]
+      const int k = kk + (lane >> 5);
+      float av[WT], bv[WT];
 #pragma unroll
-      for (int i = 0; i < 4; ++i) av[i] = As[k][ty * 4 + i];
+      for (int i = 0; i < WT; ++i) av[i] = As[k][(wm * WT + i) * 32 + (lane & 31)];
 #pragma unroll
-      for (int j = 0; j < 4; ++j) bv[j] = Bs[k][tx * 4 + j];
+      for (int j = 0; j < WT; ++j) bv[j] = Bs[k][(wn * WT + j) * 32 + (lane & 31)];
 #pragma unroll
-      for (int i = 0; i < 4; ++i)
+      for (int i = 0; i < WT; ++i)
 #pragma unroll
-        for (int j = 0; j < 4; ++j) acc[i][j] = __builtin_fmaf(av[i], bv[j], acc[i][j]);
+        for (int j = 0; j < WT; ++j)
+          acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(av[i], bv[j], acc[i][j], 0, 0, 0);
     }
     __syncthreads();
   }
+  // accumulator element r of lane l: row 8 * (r / 4) + 4 * (l / 32) + r % 4, column l % 32
 #pragma unroll
-  for (int i = 0; i < 4; ++i)
+  for (int i = 0; i < WT; ++i)
 #pragma unroll
-    for (int j = 0; j < 4; ++j) {
-      size_t r = m0 + ty * 4 + i, c = n0 + tx * 4 + j;
-      if (r < M && c < N) {
-        if (out_dtype == BQ_BF16)
-          static_cast<uint16_t*>(out)[r * N + c] = f32_to_bf16(acc[i][j]);
-        else
-          static_cast<float*>(out)[r * N + c] = acc[i][j];
+    for (int j = 0; j < WT; ++j)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        const size_t row = m0 + (wm * WT + i) * 32 + 8 * (r / 4) + 4 * (lane >> 5) + r % 4;
+        const size_t col = n0 + (wn * WT + j) * 32 + (lane & 31);
+        if (row < M && col < N) {
+          if (out_dtype == BQ_BF16)
+            static_cast<uint16_t*>(out)[row * N + col] = f32_to_bf16(acc[i][j][r]);
+          else
+            static_cast<float*>(out)[row * N + col] = acc[i][j][r];
+        }
       }
-    }
 }
 
 unsigned log2_exact(size_t v) {
@@ -558,9 +589,16 @@ bq_status launch_bf16_to_f32(const uint16_t* src, size_t n, float* dst, hipStrea
 bq_status launch_float_matmul(const void* a, int a_dtype, const void* b, int b_dtype, size_t m,
                               size_t k, size_t n, int out_dtype, void* out, hipStream_t st) {
   if (m == 0 || n == 0) return BQ_OK;
-  dim3 grid((n + 63) / 64, (m + 63) / 64), tb(256);
-  hipLaunchKernelGGL(float_matmul_kernel, grid, tb, 0, st, a, a_dtype, b, b_dtype, m, k, n,
-                     out_dtype, out);
+  // 128 x 128 tiles once they fill the chip (more reuse per byte read), 64 x 64 below
+  const bool big = ((m + 127) / 128) * ((n + 127) / 128) >= 256;
+  const size_t t = big ? 128 : 64;
+  if ((n + t - 1) / t > 0x7FFFFFFFu || (m + t - 1) / t > 65535u)
+    BQ_FAIL(BQ_ERR_SIZE, "float matmul of %zu x %zu outputs exceeds the launch grid", m, n);
+  dim3 grid(static_cast<unsigned>((n + t - 1) / t), static_cast<unsigned>((m + t - 1) / t)), tb(256);
+  if (big)
+    hipLaunchKernelGGL(float_matmul_kernel<2>, grid, tb, 0, st, a, a_dtype, b, b_dtype, m, k, n, out_dtype, out);
+  else
+    hipLaunchKernelGGL(float_matmul_kernel<1>, grid, tb, 0, st, a, a_dtype, b, b_dtype, m, k, n, out_dtype, out);
   BQ_HIP(hipGetLastError());
   return BQ_OK;
 }

@@ -936,15 +936,18 @@ static bq_status q_matmul_impl(const bq_tensor* lhs, const bq_tensor* rhs, int32
     *out = o;
     return BQ_OK;
   }
+  // A quantized lhs is dequantized (to f32 when both operands are quantized, as the reference does)
+  // and then multiplied like a float one: the weight stays packed and the matrix-core kernels run.
+  const int32_t lhs_dtype = lq ? target : lhs->dtype;
   long run = rq ? run_block(rhs->scheme, rhs->shape, rhs->rank) : -1;
-  bool fused = !lq && rq && run >= 0 && value_known(rhs->scheme.value);
+  bool fused = rq && run >= 0 && value_known(rhs->scheme.value);
   if (fused && run > 0) {
     const size_t vpl = static_cast<size_t>(num_quants(rhs->scheme.value));
     const size_t bw = static_cast<size_t>(run) / vpl;
     fused = (static_cast<size_t>(run) % vpl == 0) && bw && !(bw & (bw - 1)) && d.n % static_cast<size_t>(run) == 0;
   }
   if (fused && (d.n % static_cast<size_t>(num_quants(rhs->scheme.value)))) fused = false;
-  if (fused && !fused_matmul_ok(d.m, d.k, d.n, lhs->dtype, rhs->scheme.value,
+  if (fused && !fused_matmul_ok(d.m, d.k, d.n, lhs_dtype, rhs->scheme.value,
                                 run > 0 ? d.n / static_cast<size_t>(run) : 0))
     fused = false;
   // The fused kernels take 16-byte aligned operands: with several batches every batch's slice of
@@ -953,17 +956,23 @@ static bq_status q_matmul_impl(const bq_tensor* lhs, const bq_tensor* rhs, int32
     const size_t vbytes = rhs->scheme.store == BQ_STORE_NATIVE
                               ? d.k * d.n
                               : 4 * d.k * (d.n / static_cast<size_t>(num_quants(rhs->scheme.value)));
-    if ((d.m * d.k * dtype_size(lhs->dtype)) % 16 || (d.m * d.n * dtype_size(out_dtype)) % 16 || vbytes % 16 ||
+    if ((d.m * d.k * dtype_size(lhs_dtype)) % 16 || (d.m * d.n * dtype_size(out_dtype)) % 16 || vbytes % 16 ||
         (run > 0 && (d.k * (d.n / static_cast<size_t>(run)) * sizeof(float)) % 16))
       fused = false;
   }
 
   if (fused) {
+    bq_tensor* lf = nullptr;
+    if (lq) BQ_TRY(bq_dequantize(lhs, lhs_dtype, &lf));
+    const bq_tensor* l = lq ? lf : lhs;
     bq_tensor* o = nullptr;
-    BQ_TRY(new_float(dev, out_dtype, d.out_shape, d.rank, &o));
-    const size_t ws = bqk_q_matmul_workspace(d.m, d.k, d.n, lhs->dtype, rhs->scheme.value);
+    bq_status rc = new_float(dev, out_dtype, d.out_shape, d.rank, &o);
+    if (rc != BQ_OK) {
+      if (lf) bq_tensor_release(lf);
+      return rc;
+    }
+    const size_t ws = bqk_q_matmul_workspace(d.m, d.k, d.n, lhs_dtype, rhs->scheme.value);
     std::unique_lock<std::mutex> lock(dev->mu, std::defer_lock);
-    bq_status rc = BQ_OK;
     if (ws) {
       lock.lock();  // the split-K workspace is shared by the calls on this device
       rc = dev->ensure_workspace(ws);
@@ -975,15 +984,16 @@ static bq_status q_matmul_impl(const bq_tensor* lhs, const bq_tensor* rhs, int32
     for (size_t b = 0; b < d.batches && rc == BQ_OK; ++b) {
       size_t lb, rb;
       batch_offsets(d, b, &lb, &rb);
-      rc = bqk_q_linear(static_cast<char*>(lhs->data) + lb * d.m * d.k * dtype_size(lhs->dtype), lhs->dtype,
+      rc = bqk_q_linear(static_cast<char*>(l->data) + lb * d.m * d.k * dtype_size(lhs_dtype), lhs_dtype,
                         d.m, d.k, d.n, static_cast<char*>(rhs->data) + rb * vbytes_per_batch,
                         rhs->scales() + rb * scales_per_batch, static_cast<int32_t>(run), rhs->scheme.value,
                         rhs->scheme.store, bias, out_dtype,
                         static_cast<char*>(o->data) + b * d.m * d.n * dtype_size(out_dtype), dev->workspace,
                         dev->workspace_bytes, st);
     }
+    if (lock.owns_lock()) lock.unlock();  // (releasing a tensor takes the same mutex)
+    if (lf) bq_tensor_release(lf);         // (stream-ordered: the kernels above were enqueued first)
     if (rc != BQ_OK) {
-      if (lock.owns_lock()) lock.unlock();  // (releasing the output takes the same mutex)
       bq_tensor_release(o);
       return rc;
     }

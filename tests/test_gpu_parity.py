@@ -354,6 +354,42 @@ def test_q_matmul_batched_small_operands(dev, b, m, k, n, rhs_batched):
         assert np.abs(got - ref).max() <= tol * np.abs(ref).max()
 
 
+@pytest.mark.parametrize("m,k,n", [(1, 1, 1), (5, 7, 3), (64, 64, 64), (65, 33, 130), (512, 512, 512),
+                                   (200, 1000, 72), (1, 300, 640), (300, 24, 2112), (2100, 96, 2100)])
+def test_q_matmul_other_operand_combinations(dev, m, k, n):
+    """quantized x quantized, quantized x float, float x a weight in rectangle blocks: the
+    quantized operands are dequantized (crates/burn-backend/src/backend/ops/qtensor.rs:498-544),
+    then multiplied in f32 -- by the packed-weight kernels when the rhs is one they take, by the
+    f32 matrix-core GEMM otherwise. Yardstick: the float64 product of the dequantized operands."""
+    rng = np.random.default_rng(m * 131 + k * 17 + n)
+    a = rng.standard_normal((m, k)).astype(np.float32)
+    b = rng.standard_normal((k, n)).astype(np.float32)
+
+    def quantized(x, scheme):
+        t = QTensorOps.quantize_dynamic(FloatOps.float_from_data(x, dev), scheme)
+        q, s = unpack_blob(QTensorOps.q_into_data(t))
+        blk = list(scheme.block) if scheme.block else None
+        return t, no.dequantize(q, s, blk).astype(np.float64)
+
+    def check(out, ref, tol):
+        assert out.shape == ref.shape and out.dtype == ba.F32
+        assert np.abs(FloatOps.float_into_data(out) - ref).max() <= tol * max(np.abs(ref).max(), 1e-30)
+
+    ql, al = quantized(a, QuantScheme() if k % 4 == 0 else QuantScheme(store=QuantStore.Native))
+    packed = QuantScheme() if n % 4 == 0 else QuantScheme(store=QuantStore.Native)
+    qr, br = quantized(b, packed)
+    # (more than 32 rows against a packed weight: the prefill kernel, whose operands are bf16)
+    check(QTensorOps.q_matmul(ql, qr), al @ br, 2e-5 if (m <= 32 or n % 4) else 1e-2)
+    check(QTensorOps.q_matmul(ql, FloatOps.float_from_data(b, dev)), al @ b.astype(np.float64), 2e-5)
+    if k % 2 == 0 and n % 8 == 0:
+        qrect, brect = quantized(b, QuantScheme().per_block((2, 8)))
+        check(QTensorOps.q_matmul(FloatOps.float_from_data(a, dev), qrect), a.astype(np.float64) @ brect, 2e-5)
+        check(QTensorOps.q_matmul(ql, qrect), al @ brect, 2e-5)
+    if n % 32 == 0:
+        q4, b4 = quantized(b, QuantScheme(value=QuantValue.Q4S).per_block((32,)))
+        check(QTensorOps.q_matmul(ql, q4), al @ b4, 2e-5 if m <= 32 else 1e-2)
+
+
 def test_error_behaviour(dev):
     x = FloatOps.float_from_data(np.zeros((4, 6), np.float32), dev)
     with pytest.raises(ba.BurnqError, match="Can't store in u32"):
