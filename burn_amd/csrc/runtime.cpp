@@ -1181,12 +1181,37 @@ extern "C" bq_status bq_q_reshape(const bq_tensor* t, const size_t* shape, int32
             shape[rank - 1], nq);
   if (s.level == BQ_LEVEL_BLOCK) {
     // Only metadata moves, so the blocks must stay the same runs of the flat storage.
+    // The run is laid over the new trailing dims: whole dims while it is at least as long as they
+    // are, then a divisor of the next one. (Block extents are bytes, as in the reference's
+    // BlockSize, so a run of 256 or more has to be spread over several dims.)
     const long run = run_block(s, t->shape, t->rank);
-    if (run <= 0 || shape[rank - 1] % static_cast<size_t>(run) || run > 255)
+    size_t rem = run > 0 ? static_cast<size_t>(run) : 0;
+    uint8_t blk[BQ_MAX_RANK];
+    int used = 0;
+    for (int d = rank - 1; d >= 0 && rem > 1; --d) {
+      const size_t ext = shape[d];
+      size_t take;
+      if (rem >= ext && ext > 0 && rem % ext == 0) {
+        take = ext;
+        rem /= ext;
+      } else if (rem < ext && ext % rem == 0) {
+        take = rem;
+        rem = 1;
+      } else {
+        break;
+      }
+      if (take > 255) {
+        rem = 0;
+        break;
+      }
+      blk[used++] = static_cast<uint8_t>(take);
+    }
+    if (rem != 1)
       BQ_FAIL(BQ_ERR_UNSUPPORTED_OP,
-              "reshape of a block-quantized tensor needs blocks that are runs dividing the new last dim");
-    s.block_rank = 1;
-    s.block[0] = static_cast<uint8_t>(run);
+              "reshape of a block-quantized tensor needs blocks that stay runs of the new trailing dims");
+    if (used == 0) blk[used++] = 1;
+    s.block_rank = static_cast<uint8_t>(used);
+    for (int j = 0; j < used; ++j) s.block[j] = blk[used - 1 - j];  // (outermost of the used dims first)
   }
   bq_tensor* a = alias_of(t);
   a->rank = rank;
@@ -1199,7 +1224,10 @@ extern "C" bq_status bq_q_reshape(const bq_tensor* t, const size_t* shape, int32
 // q_permute and q_flip in one gather: output dim a reads source dim axes[a], backwards where
 // flip[axes[a]] is set. Block scales move with their blocks, as in
 // crates/burn-ndarray/src/ops/qtensor.rs:310-336 (scheme.permute_block_dims).
-static bq_status q_gather_impl(const bq_tensor* t, const int32_t* axes, const uint8_t* flip, bq_tensor** out) {
+// keep_params: the scales are copied as they are, whatever happens to the values (the reference's
+// q_flip).
+static bq_status q_gather_impl(const bq_tensor* t, const int32_t* axes, const uint8_t* flip, bq_tensor** out,
+                               bool keep_params = false) {
   const int rank = t->rank;
   size_t new_shape[BQ_MAX_RANK], old_blk[BQ_MAX_RANK], old_params[BQ_MAX_RANK];
   block_dims(t->scheme, rank, old_blk);
@@ -1218,7 +1246,7 @@ static bq_status q_gather_impl(const bq_tensor* t, const int32_t* axes, const ui
   bq_status rc = launch_q_gather(t->data, q->data, t->shape, rank, axes, flip, scheme.value,
                                  scheme.store == BQ_STORE_NATIVE, st);
   if (rc == BQ_OK) {
-    if (scheme.level == BQ_LEVEL_BLOCK) {
+    if (scheme.level == BQ_LEVEL_BLOCK && !keep_params) {
       rc = launch_f32_gather(t->scales(), q->scales(), old_params, rank, axes, flip, st);
     } else {
       hipError_t e = hipMemcpyAsync(q->scales(), t->scales(), 4 * t->num_scales, hipMemcpyDeviceToDevice, st);
@@ -1282,13 +1310,10 @@ extern "C" bq_status bq_q_flip(const bq_tensor* t, const int32_t* axes, int32_t 
     if (flip[axes[i]]) BQ_FAIL(BQ_ERR_SHAPE, "flip axis %d is repeated", axes[i]);
     flip[axes[i]] = 1;
   }
-  // The reference flips the values and keeps the parameters as they are
-  // (crates/burn-ndarray/src/ops/qtensor.rs:338-347), which only describes the flipped tensor when
-  // there is one scale; with block scales this backend declines, as burn-cubecl does for every
-  // scheme (crates/burn-cubecl/src/ops/qtensor.rs:321-323).
-  if (t->scheme.level != BQ_LEVEL_TENSOR)
-    BQ_FAIL(BQ_ERR_UNSUPPORTED_OP, "q_flip of a block-quantized tensor is not implemented by this backend");
+  // The reference flips the values and keeps the parameters as they are, block scales included
+  // (crates/burn-ndarray/src/ops/qtensor.rs:338-347): after a flip across blocks a value is
+  // dequantized with the scale of the block it lands in. Reproduced as it is.
   int32_t ident[BQ_MAX_RANK];
   for (int d = 0; d < t->rank; ++d) ident[d] = d;
-  return q_gather_impl(t, ident, flip, out);
+  return q_gather_impl(t, ident, flip, out, /*keep_params=*/true);
 }

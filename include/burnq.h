@@ -225,8 +225,9 @@ bq_status bq_q_reshape(const bq_tensor* t, const size_t* shape, int32_t rank, bq
  * dense tensor (the block of the scheme is permuted with the axes, so a [1, 32] block becomes
  * [32, 1] under a transpose). An axis out of bounds or repeated, which the reference panics on,
  * returns BQ_ERR_SHAPE, as does a packed result whose last dim is not a whole number of words.
- * q_flip of a block-quantized tensor returns BQ_ERR_UNSUPPORTED_OP: the reference keeps the
- * parameters in place there, which only describes the flipped tensor when there is one scale. */
+ * q_flip flips the values and keeps every parameter where it is, block scales included, as the
+ * reference does (burn-ndarray/src/ops/qtensor.rs:338-347): a value flipped into another block
+ * is dequantized with that block's scale. */
 bq_status bq_q_swap_dims(const bq_tensor* t, int32_t dim1, int32_t dim2, bq_tensor** out);
 bq_status bq_q_permute(const bq_tensor* t, const int32_t* axes, int32_t rank, bq_tensor** out);
 bq_status bq_q_flip(const bq_tensor* t, const int32_t* axes, int32_t n_axes, bq_tensor** out);

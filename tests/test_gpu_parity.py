@@ -417,8 +417,24 @@ def test_q_reshape_is_metadata_only(dev):
     assert r.shape == (4, 256) and r.data_ptr == tq.data_ptr
     d = FloatOps.float_into_data(QTensorOps.dequantize(r))
     assert d.tobytes() == d_ref.reshape(4, 256).tobytes()
+    # a last dim shorter than the block: the run of 32 becomes a [2, 16] block
+    r = QTensorOps.q_reshape(tq, (64, 16))
+    assert r.scheme.block == (2, 16) and r.data_ptr == tq.data_ptr
+    assert FloatOps.float_into_data(QTensorOps.dequantize(r)).tobytes() == d_ref.reshape(64, 16).tobytes()
+    t6, _, _, d6 = check_quantize_dynamic(dev, awkward((6, 64), 9), scheme)
     with pytest.raises(ba.BurnqError):
-        QTensorOps.q_reshape(tq, (64, 16))   # blocks of 32 would no longer divide the last dim
+        QTensorOps.q_reshape(t6, (8, 48))    # runs of 32 do not tile rows of 48
+    # runs of 256 values and more do not fit one block extent (a byte): spread over two dims
+    big = QuantScheme().per_block((2, 128))
+    tb, _, _, db = check_quantize_dynamic(dev, awkward((4, 2, 128), 10), big)
+    r = QTensorOps.q_reshape(tb, (8, 128))
+    assert r.scheme.block == (2, 128)
+    assert FloatOps.float_into_data(QTensorOps.dequantize(r)).tobytes() == db.reshape(8, 128).tobytes()
+    r = QTensorOps.q_reshape(tb, (2, 8, 64))
+    assert r.scheme.block == (4, 64)
+    assert FloatOps.float_into_data(QTensorOps.dequantize(r)).tobytes() == db.reshape(2, 8, 64).tobytes()
+    with pytest.raises(ba.BurnqError):
+        QTensorOps.q_reshape(tb, (2, 512))   # one extent of 256
     same = QTensorOps.q_to_device(tq, dev)
     assert QTensorOps.q_into_data(same).bytes.tobytes() == QTensorOps.q_into_data(tq).bytes.tobytes()
 
@@ -483,13 +499,16 @@ def test_q_permute_matches_oracle(dev, value, store, block, shape, axes):
     d = FloatOps.float_into_data(QTensorOps.dequantize(tp))
     assert d.tobytes() == np.transpose(FloatOps.float_into_data(QTensorOps.dequantize(tq)), axes).copy().tobytes()
     assert d.tobytes() == no.dequantize(qp, sp, bp).tobytes()
-    if block is None:
-        f = QTensorOps.q_flip(tq, [0, len(shape) - 1])
-        qf, sf = no.q_flip(q, s, [0, len(shape) - 1])
-        assert (unpack_blob(QTensorOps.q_into_data(f))[0] == qf).all()
-    else:
-        with pytest.raises(ba.BurnqError):
-            QTensorOps.q_flip(tq, [0])
+    # q_flip: the values are flipped, the parameters stay where they are -- block scales too, as in
+    # the reference (crates/burn-ndarray/src/ops/qtensor.rs:338-347)
+    for flip_axes in ([0, len(shape) - 1], [len(shape) - 1], [0]):
+        f = QTensorOps.q_flip(tq, flip_axes)
+        qf, sf = no.q_flip(q, s, flip_axes)
+        got_q, got_s = unpack_blob(QTensorOps.q_into_data(f))
+        assert (got_q == qf).all()
+        assert np.asarray(got_s, np.float32).tobytes() == np.asarray(sf, np.float32).tobytes()
+        assert FloatOps.float_into_data(QTensorOps.dequantize(f)).tobytes() == \
+            no.dequantize(qf, sf, list(block) if block else None).tobytes()
 
 
 def test_hip_graph_replays_match_eager(dev):
