@@ -52,7 +52,9 @@ constexpr int kSplitWaves = kGroups * kKWays;
 constexpr int kSplitThreads = kSplitWaves * kWave;  // 512
 constexpr int kUnits = 4;                           // blocks of 32 columns per wave
 constexpr int kStepRows = 32;                       // k rows per MFMA
-constexpr int kDepth = 2;                           // steps of loads in flight per wave
+// steps of loads in flight per wave (3 and 4 were slower by 1.5 and 2 us: the burst of first loads
+// is that much larger, and every wave's first step arrives behind all of it)
+constexpr int kDepth = 2;
 constexpr int kGroupCols = kUnits * 32;             // 128
 constexpr int kTileCols = kGroups * kGroupCols;     // 512 columns per workgroup
 constexpr int kMaxSlice = 512;                      // k rows per workgroup (activations in LDS: 16 x 516 floats)
@@ -109,6 +111,10 @@ qsplit_kernel(const void* __restrict__ x, const uint32_t* __restrict__ w, const 
   constexpr int RPI = kWave / LPR;           // rows per load instruction: 8 or 16
   constexpr int NLOAD = kStepRows / RPI;     // load instructions per step: 4 or 2
   constexpr uint32_t ROT = ROW_B / 4;        // slot rotation per 8 rows
+  // Two measured choices for Q8S (the Q4S kernels move half the bytes and gain nothing from either):
+  // the first weight loads wait for the activations, and a wave's priority falls with its progress.
+  constexpr bool kLateFetch = VPL == 4;
+  constexpr bool kProgressPriority = VPL == 4;
   const int tid = threadIdx.x;
   const int lane = tid & (kWave - 1);
   const int wave = __builtin_amdgcn_readfirstlane(tid / kWave);
@@ -202,16 +208,28 @@ qsplit_kernel(const void* __restrict__ x, const uint32_t* __restrict__ w, const 
   // against a zero weight), Q4S weights are converted to their true values instead of the offset
   // patterns (inf * (q + 136) - inf * 136 is NaN), and the padded step past the end is skipped
   // (inf * 0). Finite slices never execute any of it.
+  // (-1, 0) and (0, -1) as bf16 pairs, kept in registers the compiler cannot see through: written
+  // as constants, (-1, 0) becomes the inline operand -1.0, which this instruction reads as the 32-bit
+  // float -- the pair (0, -1).
+  uint32_t minus_lo = 0x0000BF80u, minus_hi = 0xBF800000u;
+  asm volatile("" : "+s"(minus_lo), "+s"(minus_hi));
   auto split = [&](auto G, const float* t, uint32_t* hi, uint32_t* lo) {
     constexpr bool guard = decltype(G)::value;
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
       hi[i] = pack_bf16(t[2 * i], t[2 * i + 1]);
-      const float h0 = as_float(hi[i] << 16), h1 = as_float(hi[i] & 0xFFFF0000u);
-      float d0 = t[2 * i] - h0, d1 = t[2 * i + 1] - h1;
+      float d0, d1;
       if (guard) {
-        d0 = (as_bits(h0) & 0x7F800000u) == 0x7F800000u ? 0.0f : d0;
-        d1 = (as_bits(h1) & 0x7F800000u) == 0x7F800000u ? 0.0f : d1;
+        const float h0 = as_float(hi[i] << 16), h1 = as_float(hi[i] & 0xFFFF0000u);
+        d0 = (as_bits(h0) & 0x7F800000u) == 0x7F800000u ? 0.0f : t[2 * i] - h0;
+        d1 = (as_bits(h1) & 0x7F800000u) == 0x7F800000u ? 0.0f : t[2 * i + 1] - h1;
+      } else {
+        // t - hi straight from the packed pair: v_dot2_f32_bf16 against (-1, 0) and (0, -1) adds
+        // -hi to t in one instruction each (the difference has at most 16 significant bits, so
+        // it is exact), where unpacking the halves first costs a shift and a mask more per pair
+        const bf16x2 h = __builtin_bit_cast(bf16x2, hi[i]);
+        d0 = __builtin_amdgcn_fdot2_f32_bf16(h, __builtin_bit_cast(bf16x2, minus_lo), t[2 * i], false);
+        d1 = __builtin_amdgcn_fdot2_f32_bf16(h, __builtin_bit_cast(bf16x2, minus_hi), t[2 * i + 1], false);
       }
       lo[i] = pack_bf16(d0, d1);
     }
@@ -315,9 +333,8 @@ qsplit_kernel(const void* __restrict__ x, const uint32_t* __restrict__ w, const 
     }
   };
 
-  // The activation loads go first: loads return in order, and the first multiply needs the
-  // activations and the first step of weights only, not everything that is in flight behind them.
-  // (Buffer loads: rows past M and columns past K read as zero through the range check.)
+  // The activations of the slice, through registers into LDS. (Buffer loads: rows past M and
+  // columns past K read as zero through the range check.)
   int bad = 0;
   {
     constexpr uint32_t XB = X_BF16 ? 2u : 4u;  // bytes per activation
@@ -339,9 +356,11 @@ qsplit_kernel(const void* __restrict__ x, const uint32_t* __restrict__ w, const 
       }
     }
     __builtin_amdgcn_sched_barrier(0);
+    if (!kLateFetch) {
 #pragma unroll
-    for (int b = 0; b < kDepth; ++b) fetch(b, b);
-    __builtin_amdgcn_sched_barrier(0);
+      for (int b = 0; b < kDepth; ++b) fetch(b, b);
+      __builtin_amdgcn_sched_barrier(0);
+    }
 #pragma unroll
     for (int i = 0; i < kFillVecs * MT; ++i) {
       const uint32_t idx = static_cast<uint32_t>(tid) + static_cast<uint32_t>(i) * kSplitThreads;
@@ -353,6 +372,16 @@ qsplit_kernel(const void* __restrict__ x, const uint32_t* __restrict__ w, const 
     }
   }
   const bool nonfinite = __syncthreads_or(bad) != 0;
+  // Q8S: the first weight loads go out only now, with the activations in LDS. Issued ahead of
+  // them (to overlap the two round trips), the weights of all the workgroups fill the memory
+  // system's queues and the small activation loads come back 3 us later instead of 1 us: the first
+  // multiply of every wave waits for them, and the kernel took about 1 us longer that way (measured
+  // with per-wave timestamps on the 4096 x 14336 weight, as are the other figures in this file).
+  if (kLateFetch) {
+#pragma unroll
+    for (int b = 0; b < kDepth; ++b) fetch(b, b);
+    __builtin_amdgcn_sched_barrier(0);
+  }
 
   // (scheduling barriers: left alone, the compiler sinks a step's loads below the other step's
   // MFMAs to save registers, which puts the load latency in series with the arithmetic)
@@ -360,6 +389,17 @@ qsplit_kernel(const void* __restrict__ x, const uint32_t* __restrict__ w, const 
     for (int s0 = 0; s0 < steps; s0 += kDepth) {
 #pragma unroll
       for (int b = 0; b < kDepth; ++b) {
+        // Two waves share a SIMD (one of each half of the K slice), and the arbiter prefers the
+        // older: left alone, that one runs ahead and the other finishes 3 us after it, alone on
+        // the SIMD, with nothing to cover its waits. The priority falls with a wave's progress, so
+        // the wave that is behind goes first and both finish together (1 us sooner).
+        if (kProgressPriority) {
+          const int quarter = (s0 + b) * 4 / steps;
+          if (quarter <= 0) __builtin_amdgcn_s_setprio(3);
+          else if (quarter == 1) __builtin_amdgcn_s_setprio(2);
+          else if (quarter == 2) __builtin_amdgcn_s_setprio(1);
+          else __builtin_amdgcn_s_setprio(0);
+        }
         multiply(std::false_type{}, b, s0 + b);
         __builtin_amdgcn_sched_barrier(0);
         fetch(b, s0 + b + kDepth);
