@@ -371,6 +371,40 @@ def run_c4(ba, dev, steps, warmup, cpu):
 C5_N = 14336  # weight columns of C5; --c5-n runs the same product at another width (tile-count studies)
 
 
+VENDOR_GEMM = r"""
+import sys, torch
+m, k, n = (int(v) for v in sys.argv[1:4])
+a = [torch.randn(m, k, device="cuda:0", dtype=torch.bfloat16) for _ in range(4)]
+b = [torch.randn(k, n, device="cuda:0", dtype=torch.bfloat16) * 0.02 for _ in range(4)]
+for i in range(12): a[i % 4] @ b[i % 4]
+torch.cuda.synchronize()
+s, e = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+best = 1e9
+for rep in range(5):
+    s.record()
+    for i in range(20): a[i % 4] @ b[i % 4]
+    e.record(); torch.cuda.synchronize()
+    best = min(best, s.elapsed_time(e) / 20)
+print(best)
+"""
+
+
+def vendor_gemm_yardstick(m, k, n):
+    """A plain bf16 x bf16 -> bf16 GEMM of the same shape through torch.matmul (the vendor's GEMM
+    library), weights already dequantized and row-major [K, N] as here: what the matrix pipe yields
+    on this box with no dequantization to do. A yardstick beside the roofline, not part of the
+    product; run in a process of its own, None if torch is not usable there."""
+    import subprocess
+    try:
+        p = subprocess.run([sys.executable, "-c", VENDOR_GEMM, str(m), str(k), str(n)], capture_output=True, text=True,
+                           timeout=180)
+        ms = float(p.stdout.strip().splitlines()[-1])
+    except Exception:
+        return None
+    return {"ms": round(ms, 4), "TFLOP/s": round(2.0 * m * k * n / ms / 1e9, 1),
+            "what": "torch.matmul, bf16 [M,K] @ bf16 row-major [K,N] -> bf16, best of 5 runs of 20 calls over 4 operand pairs"}
+
+
 def run_c5(ba, dev, steps, warmup, cpu):
     from burn_amd import FloatOps, QTensorOps, QuantValue
     from oracle import c_oracle as co
@@ -422,6 +456,7 @@ def run_c5(ba, dev, steps, warmup, cpu):
            "roofline": roofline("mfma", tf, BF16_PEAK_TFLOPS, "TFLOP/s", "qgemm_kernel<8,256,f32>", ev),
            "ms_eager_submission": ev_eager, "timing": "HIP graph of 8 calls over 4 weight copies; ms per call",
            "linear_with_bias_ms_eager": ev_lin, "bf16_output_ms_eager": ev_h}
+    out["vendor_bf16_gemm"] = vendor_gemm_yardstick(m, k, n)
     if cpu:
         osch = co.Scheme.make(co.Q4S, [32], co.STORE_PACKED_U32)
         q = co.unpack_u32(values.view(np.uint32), (k, n), co.Q4S)

@@ -77,6 +77,7 @@ SIGNATURES = {
     "bq_device_stream": (_vp, [_vp]),
     "bq_device_trim": (_i32, [_vp]),
     "bq_device_set_validate": (_i32, [_vp, _i32]),
+    "bq_device_set_f32_matmul_exact": (_i32, [_vp, _i32]),
     "bq_timer_start": (_i32, [_vp]),
     "bq_timer_stop": (_i32, [_vp, C.POINTER(C.c_float)]),
     "bq_graph_begin_capture": (_i32, [_vp]),

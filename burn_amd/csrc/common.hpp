@@ -71,6 +71,7 @@ struct bq_device {
   int num_cus = 256;
   size_t lds_limit = 64 * 1024;                   // largest dynamic LDS request a launch may make
   std::atomic<bool> validate{false};              // bq_device_set_validate
+  std::atomic<bool> f32_matmul_exact{false};  // bq_device_set_f32_matmul_exact
   uint32_t* validate_cells = nullptr;             // 4 device counters of the validate mode
 
   // *actual receives the size of the block handed out (at least `bytes`); pass it to release().

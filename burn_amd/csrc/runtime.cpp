@@ -316,6 +316,12 @@ extern "C" bq_status bq_device_set_validate(bq_device* dev, int32_t on) {
   return BQ_OK;
 }
 
+extern "C" bq_status bq_device_set_f32_matmul_exact(bq_device* dev, int32_t on) {
+  BQ_NOTNULL(dev);
+  dev->f32_matmul_exact.store(on != 0);
+  return BQ_OK;
+}
+
 extern "C" bq_status bqk_lds_request_status(size_t bytes, size_t device_limit) {
   return lds_request_status(bytes, device_limit, "kernel");
 }
@@ -947,6 +953,8 @@ static bq_status q_matmul_impl(const bq_tensor* lhs, const bq_tensor* rhs, int32
     fused = (static_cast<size_t>(run) % vpl == 0) && bw && !(bw & (bw - 1)) && d.n % static_cast<size_t>(run) == 0;
   }
   if (fused && (d.n % static_cast<size_t>(num_quants(rhs->scheme.value)))) fused = false;
+  // (f32 activations, more than 32 rows: the fast kernels round to bf16; the device may ask for f32)
+  if (fused && lhs_dtype == BQ_F32 && d.m > 32 && dev->f32_matmul_exact.load()) fused = false;
   if (fused && !fused_matmul_ok(d.m, d.k, d.n, lhs_dtype, rhs->scheme.value,
                                 run > 0 ? d.n / static_cast<size_t>(run) : 0))
     fused = false;

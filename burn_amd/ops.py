@@ -49,6 +49,11 @@ class Device:
         quotient (NaN input or scale, infinite input against an infinite scale)."""
         check(lib().bq_device_set_validate(self.handle, 1 if on else 0))
 
+    def set_f32_matmul_exact(self, on: bool):
+        """f32 activations with more than 32 rows: multiply the reference's way (dequantize to
+        f32, f32 product) instead of the bf16 matrix-core kernel."""
+        check(lib().bq_device_set_f32_matmul_exact(self.handle, 1 if on else 0))
+
     @property
     def stream(self) -> int:
         return lib().bq_device_stream(self.handle) or 0

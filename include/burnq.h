@@ -107,6 +107,14 @@ bq_status bq_device_trim(bq_device* dev);
  * stream (a debugging aid; refused during graph capture). Off, such inputs give unspecified
  * integers. */
 bq_status bq_device_set_validate(bq_device* dev, int32_t on);
+/* f32 activations against a quantized weight keep at least 16 significant bits per product up to
+ * 32 rows; from 33 rows on the fast kernel rounds them (and s * q) to bf16, about 2e-3 of the
+ * largest output, inside the 1e-2 the reference's own tests allow
+ * (crates/burn-backend-tests/tests/tensor/float/quantization/ops/matmul.rs) but far from its f32
+ * sgemm. on != 0 makes q_matmul / q_linear on this device multiply such products the reference's
+ * way instead -- dequantize to f32, f32 matrix product -- at a fraction of the speed. Off by
+ * default. No counterpart in the reference. */
+bq_status bq_device_set_f32_matmul_exact(bq_device* dev, int32_t on);
 /* HIP-event stopwatch on the context's stream (what Backend::sync-bracketed benches measure,
  * without the host round trip): start, enqueue work, stop -> elapsed milliseconds. */
 bq_status bq_timer_start(bq_device* dev);

@@ -15,7 +15,7 @@ from conftest import burn_approx_eq
 pytestmark = pytest.mark.gpu
 
 import burn_amd as ba  # noqa: E402
-from burn_amd import FloatOps, QTensorOps, QuantScheme, QuantStore, QuantValue, TensorData  # noqa: E402
+from burn_amd import FloatOps, ModuleOps, QTensorOps, QuantScheme, QuantStore, QuantValue, TensorData  # noqa: E402
 from burn_amd.quantization import ScaleDtype  # noqa: E402
 
 VAL = {QuantValue.Q8S: (co.Q8S, "Q8S"), QuantValue.Q4S: (co.Q4S, "Q4S"), QuantValue.Q2S: (co.Q2S, "Q2S")}
@@ -388,6 +388,38 @@ def test_q_matmul_other_operand_combinations(dev, m, k, n):
     if n % 32 == 0:
         q4, b4 = quantized(b, QuantScheme(value=QuantValue.Q4S).per_block((32,)))
         check(QTensorOps.q_matmul(ql, q4), al @ b4, 2e-5 if m <= 32 else 1e-2)
+
+
+@pytest.mark.parametrize("value", [QuantValue.Q8S, QuantValue.Q4S])
+def test_f32_matmul_exact_setting_removes_the_step_at_33_rows(dev, value):
+    """f32 activations x a packed weight: up to 32 rows the products keep 16 significant bits;
+    from 33 on the fast kernel rounds to bf16 (about 2e-3, inside the 1e-2 bound) unless the
+    device is told to multiply in f32, as the reference's dequantize + sgemm does."""
+    rng = np.random.default_rng(33)
+    m, k, n = 96, 1024, 640
+    w = (rng.standard_normal((k, n)) * 0.05).astype(np.float32)
+    x = rng.standard_normal((m, k)).astype(np.float32)
+    bias = rng.standard_normal(n).astype(np.float32)
+    tq = QTensorOps.quantize_dynamic(FloatOps.float_from_data(w, dev), QuantScheme(value=value).per_block((32,)))
+    q, s = unpack_blob(QTensorOps.q_into_data(tq))
+    ref = no.q_matmul_f64(x, q, s, [32])
+    xt = FloatOps.float_from_data(x, dev)
+
+    def rel(y, r):
+        return np.abs(FloatOps.float_into_data(y) - r).max() / np.abs(r).max()
+
+    fast = rel(QTensorOps.q_matmul(xt, tq), ref)
+    assert 1e-4 < fast <= 1e-2, fast                   # the bf16 kernel: the step is there
+    dev.set_f32_matmul_exact(True)
+    try:
+        assert rel(QTensorOps.q_matmul(xt, tq), ref) <= 2e-6
+        y = ModuleOps.linear(xt, tq, FloatOps.float_from_data(bias, dev))
+        assert rel(y, ref + bias[None, :].astype(np.float64)) <= 2e-6
+        # 32 rows and fewer are untouched by the setting
+        small = rel(QTensorOps.q_matmul(FloatOps.float_from_data(x[:32], dev), tq), ref[:32])
+    finally:
+        dev.set_f32_matmul_exact(False)
+    assert small <= 2e-5 and small == rel(QTensorOps.q_matmul(FloatOps.float_from_data(x[:32], dev), tq), ref[:32])
 
 
 def test_error_behaviour(dev):
@@ -1318,6 +1350,10 @@ def test_q_matmul_and_linear_random_configurations(dev, seed):
             got = ba.f32_from_bf16_bits(got).reshape(m, n)
         err = np.abs(got - ref).max() / max(np.abs(ref).max(), 1e-6)
         assert err <= (2e-2 if y.dtype == ba.BF16 else 1e-2), f"{case}: {err}"
+        # burn's elementwise rule where the path keeps f32 activations (M <= 16, f32 in and out);
+        # with bf16-rounded weights or outputs an element near zero can miss the 1e-2 floor honestly
+        if dt == ba.F32 and y.dtype == ba.F32 and m <= 16:
+            assert burn_approx_eq(got, ref, 1e-2, 1e-2).all(), case
 
 def test_more_than_2_pow_31_elements(dev):
     """[33792, 65536] f32 (2.2e9 elements, 8.9 GB): every index past 2^31 must land where the
