@@ -249,6 +249,7 @@ qsplit_kernel(const void* __restrict__ x, const uint32_t* __restrict__ w, const 
     // through the wave's slot (LDS runs a wave's instructions in order: no barrier)
 #pragma unroll
     for (int i = 0; i < NLOAD; ++i) *reinterpret_cast<vuint4*>(slot + slot_wr[i]) = wl[buf][i];
+    const vuint4 sqv = sq[buf];
     uint32_t wq[kUnits][8];
 #pragma unroll
     for (int u = 0; u < kUnits; ++u)
@@ -256,7 +257,7 @@ qsplit_kernel(const void* __restrict__ x, const uint32_t* __restrict__ w, const 
       for (int r = 0; r < 8; ++r) wq[u][r] = *reinterpret_cast<const uint32_t*>(slot + slot_rd[u] + ROW_B * r);
     uint32_t hi[MT][4], lo[MT][4];
     if (PK) {
-      const uint32_t a = sq[buf].x, b = sq[buf].y;
+      const uint32_t a = sqv.x, b = sqv.y;
       const float sr[8] = {quad_lane<0>(a), quad_lane<1>(a), quad_lane<2>(a), quad_lane<3>(a),
                            quad_lane<0>(b), quad_lane<1>(b), quad_lane<2>(b), quad_lane<3>(b)};
       float v[8];
@@ -276,7 +277,7 @@ qsplit_kernel(const void* __restrict__ x, const uint32_t* __restrict__ w, const 
 #pragma unroll
     for (int u = 0; u < kUnits; ++u) {
       if (!PER_TENSOR && !PK) {
-        const uint32_t sv = sq[buf][u >> SB];
+        const uint32_t sv = sqv[u >> SB];
         const float sr[8] = {row_lane<0>(sv), row_lane<1>(sv), row_lane<2>(sv), row_lane<3>(sv),
                              row_lane<4>(sv), row_lane<5>(sv), row_lane<6>(sv), row_lane<7>(sv)};
 #pragma unroll
