@@ -35,7 +35,8 @@ class CScheme(C.Structure):
         ("store", C.c_uint8),
         ("scale_dtype", C.c_uint8),
         ("block_rank", C.c_uint8),
-        ("reserved", C.c_uint8 * 3),
+        ("tensor_scale", C.c_uint8),
+        ("reserved", C.c_uint8 * 2),
         ("block", C.c_uint8 * MAX_RANK),
     ]
 
@@ -102,6 +103,7 @@ SIGNATURES = {
     "bq_q_from_data": (_i32, [_vp, _vp, _sz, _psz, _i32, _ps, _pvp]),
     "bq_q_into_data": (_i32, [_vp, _vp, _sz, _psz]),
     "bq_quantize": (_i32, [_vp, _ps, _vp, _pvp]),
+    "bq_quantize_two_level": (_i32, [_vp, C.POINTER(CScheme), _vp, _vp, _pvp]),
     "bq_quantize_dynamic": (_i32, [_vp, _ps, _pvp]),
     "bq_dequantize": (_i32, [_vp, _i32, _pvp]),
     "bq_q_matmul": (_i32, [_vp, _vp, _pvp]),

@@ -94,6 +94,7 @@ struct bq_tensor {
   size_t value_bytes = 0;        // dense bytes of the values region (wire size)
   size_t scales_offset = 0;
   size_t num_scales = 0;
+  size_t wire_offset = 0;        // two-level schemes: [per-tensor scale][block scales as stored], f32
   bq_tensor* base = nullptr;     // shares the memory of another handle (reshape / to_device)
 
   size_t numel() const {
@@ -104,6 +105,8 @@ struct bq_tensor {
   float* scales() const {
     return reinterpret_cast<float*>(static_cast<char*>(data) + scales_offset);
   }
+  float* wire_global() const { return reinterpret_cast<float*>(static_cast<char*>(data) + wire_offset); }
+  float* wire_scales() const { return wire_global() + 1; }
 };
 
 // ---- kernel launchers implemented in the .hip files (all enqueue on `stream`) ------------------
@@ -127,6 +130,12 @@ bq_status launch_quantize_run_block(const float* x, size_t n, int block, const f
                                     int value, int store, void* values, int scale_dtype, hipStream_t stream);
 // dst[i] = scale_to_dtype(src[i]); f32 scales <-> their 2-byte wire form (f16 / bf16).
 bq_status launch_round_scales(const float* src, float* dst, size_t n, int scale_dtype, hipStream_t stream);
+// Two-level schemes. split: `scales` holds the f32 block scales of a quantize_dynamic and `cells` the
+// partial maxima over them (bqk_absmax_f32); on return scales[i] = global * stored[i], the scale
+// the kernels use. times_global: the same product from a stored pair.
+bq_status launch_two_level_split(float* scales, size_t n, const uint32_t* cells, int scale_dtype, float* global_out,
+                                 float* stored, hipStream_t stream);
+bq_status launch_scales_times_global(const float* stored, const float* global, size_t n, float* scales, hipStream_t stream);
 bq_status launch_scales_to_wire(const float* src, void* dst, size_t n, int scale_dtype, hipStream_t stream);
 bq_status launch_scales_from_wire(const void* src, float* dst, size_t n, int scale_dtype, hipStream_t stream);
 bq_status launch_dequantize_rect(const void* values, const size_t* shape, int rank,

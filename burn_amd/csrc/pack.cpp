@@ -165,8 +165,8 @@ int dtype_from_name(const std::string& s) {
 }
 
 void write_scheme(CborWriter& w, const bq_scheme& s) {
-  w.map(5);
-  w.text("value"); w.text(s.value == BQ_Q8S ? "Q8S" : "Q4S");
+  w.map(s.tensor_scale ? 6 : 5);
+  w.text("value"); w.text(s.value == BQ_Q8S ? "Q8S" : s.value == BQ_Q4S ? "Q4S" : "Q2S");
   w.text("level");
   if (s.level == BQ_LEVEL_TENSOR) { w.text("Tensor"); }
   else { w.map(1); w.text("Block"); w.array(s.block_rank); for (int i = 0; i < s.block_rank; ++i) w.uint(s.block[i]); }
@@ -174,6 +174,7 @@ void write_scheme(CborWriter& w, const bq_scheme& s) {
   if (s.store == BQ_STORE_NATIVE) { w.text("Native"); } else { w.map(1); w.text("PackedU32"); w.uint(0); }
   w.text("scale_dtype"); w.text(s.scale_dtype == BQ_SCALE_F32 ? "F32" : s.scale_dtype == BQ_SCALE_F16 ? "F16" : "BF16");
   w.text("mode"); w.text("Symmetric");
+  if (s.tensor_scale) { w.text("tensor_scale"); w.text("F32"); }  // two-level: a per-tensor f32 scale on top
 }
 
 bool read_scheme(const Cbor& c, bq_scheme* s) {
@@ -181,7 +182,12 @@ bool read_scheme(const Cbor& c, bq_scheme* s) {
   memset(s, 0, sizeof(*s));
   const Cbor *value = c.get("value"), *level = c.get("level"), *store = c.get("store"), *sd = c.get("scale_dtype");
   if (!value || !level || !store || !sd || value->kind != Cbor::Text || sd->kind != Cbor::Text) return false;
-  if (value->s == "Q8S") s->value = BQ_Q8S; else if (value->s == "Q4S") s->value = BQ_Q4S; else return false;
+  if (value->s == "Q8S") s->value = BQ_Q8S; else if (value->s == "Q4S") s->value = BQ_Q4S;
+  else if (value->s == "Q2S") s->value = BQ_Q2S; else return false;
+  if (const Cbor* ts = c.get("tensor_scale")) {
+    if (ts->kind != Cbor::Text || ts->s != "F32") return false;
+    s->tensor_scale = 1;
+  }
   if (sd->s == "F32") s->scale_dtype = BQ_SCALE_F32; else if (sd->s == "F16") s->scale_dtype = BQ_SCALE_F16;
   else if (sd->s == "BF16") s->scale_dtype = BQ_SCALE_BF16; else return false;
   if (level->kind == Cbor::Text && level->s == "Tensor") {

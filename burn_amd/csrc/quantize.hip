@@ -568,6 +568,56 @@ bq_status launch_scale_from_cells(const uint32_t* cells, int value, int sdt, flo
   return BQ_OK;
 }
 
+// ---- two-level schemes ---------------------------------------------------------------------------
+namespace {
+
+// normalize_scales (crates/burn-backend/src/quantization/scheme.rs:106-134) and what NdArray::quantize
+// does with its result (crates/burn-ndarray/src/ops/qtensor.rs:90-101,519-531), one IEEE operation
+// per step as there: global = max(scales) / dtype_max, not below the smallest normal f32; a block
+// scale is stored as scale_to_dtype(scale / global) and the block is quantized against
+// global * that. `cells` hold the partial maxima of the scales (they are not negative).
+__global__ void __launch_bounds__(kThreads)
+two_level_split_kernel(float* __restrict__ scales, size_t n, const uint32_t* __restrict__ cells, float dtype_max, int sdt,
+                       float* __restrict__ global_out, float* __restrict__ stored) {
+  const float top = absmax_from_cells(cells);
+  const float global = fmaxf(top / dtype_max, 1.17549435e-38f);
+  if (blockIdx.x == 0 && threadIdx.x == 0) global_out[0] = global;
+  const size_t i = static_cast<size_t>(blockIdx.x) * kThreads + threadIdx.x;
+  if (i < n) {
+    const float st = scale_round_up(scales[i] / global, sdt);
+    stored[i] = st;
+    scales[i] = global * st;
+  }
+}
+
+__global__ void scales_times_global_kernel(const float* __restrict__ stored, const float* __restrict__ global, size_t n,
+                                           float* __restrict__ scales) {
+  const size_t i = static_cast<size_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+  if (i < n) scales[i] = global[0] * stored[i];
+}
+
+}  // namespace
+
+bq_status launch_two_level_split(float* scales, size_t n, const uint32_t* cells, int sdt, float* global_out, float* stored,
+                                 hipStream_t st) {
+  if (sdt != BQ_SCALE_F16)
+    BQ_FAIL(BQ_ERR_UNSUPPORTED_SCHEME,
+            "block scales of this dtype reach f32's range, which a per-tensor scale cannot absorb (f16 block scales can)");
+  if (n == 0) return BQ_OK;
+  hipLaunchKernelGGL(two_level_split_kernel, dim3(static_cast<unsigned>((n + kThreads - 1) / kThreads)), dim3(kThreads), 0, st,
+                     scales, n, cells, 65504.0f, sdt, global_out, stored);
+  BQ_HIP(hipGetLastError());
+  return BQ_OK;
+}
+
+bq_status launch_scales_times_global(const float* stored, const float* global, size_t n, float* scales, hipStream_t st) {
+  if (n == 0) return BQ_OK;
+  hipLaunchKernelGGL(scales_times_global_kernel, dim3(static_cast<unsigned>((n + 255) / 256)), dim3(256), 0, st, stored, global,
+                     n, scales);
+  BQ_HIP(hipGetLastError());
+  return BQ_OK;
+}
+
 bq_status launch_round_scales(const float* src, float* dst, size_t n, int sdt, hipStream_t st) {
   if (n == 0) return BQ_OK;
   hipLaunchKernelGGL(round_scales_kernel, dim3(static_cast<unsigned>((n + 255) / 256)), dim3(256), 0, st, src, dst, n, sdt);

@@ -60,6 +60,8 @@ static size_t value_bytes(const bq_scheme& s, const size_t* shape, int rank) {
 
 // scale_size (crates/burn-std/src/tensor/quantization.rs:409-416): bytes per stored scale on the wire.
 static size_t scale_size(const bq_scheme& s) { return s.scale_dtype == BQ_SCALE_F32 ? 4 : 2; }
+// global_scale_size (same file): the f32 per-tensor scale a two-level scheme stores behind its block scales.
+static size_t global_size(const bq_scheme& s) { return s.tensor_scale ? 4 : 0; }
 
 // What the backend accepts: the same conditions under which the reference backends panic.
 // `storable`: also require what a packed device tensor needs (whole words along the last dim). The
@@ -72,6 +74,8 @@ static bq_status check_scheme(const bq_scheme& s, const size_t* shape, int rank,
     BQ_FAIL(BQ_ERR_UNSUPPORTED_SCHEME, "scale dtype %d is not supported (f32, f16 and bf16 are)", s.scale_dtype);
   if (s.level != BQ_LEVEL_TENSOR && s.level != BQ_LEVEL_BLOCK)
     BQ_FAIL(BQ_ERR_UNSUPPORTED_SCHEME, "unknown quantization level %d", s.level);
+  if (s.tensor_scale > 1 || (s.tensor_scale && s.level != BQ_LEVEL_BLOCK))
+    BQ_FAIL(BQ_ERR_UNSUPPORTED_SCHEME, "a per-tensor scale on top (tensor_scale = %d) goes with block scales, as f32", s.tensor_scale);
   if (s.store == BQ_STORE_NATIVE) {
     if (s.value != BQ_Q8S) BQ_FAIL(BQ_ERR_UNSUPPORTED_SCHEME, "Can't store native sub-byte values");
   } else if (s.store == BQ_STORE_PACKED_U32) {
@@ -446,8 +450,14 @@ static bq_status new_quantized(bq_device* dev, const bq_scheme& scheme, const si
   t->value_bytes = value_bytes(scheme, shape, rank);
   t->num_scales = num_params(scheme, shape, rank);
   t->scales_offset = round_up(t->value_bytes, 256);
-  bq_status s = dev->alloc(round_up(t->scales_offset + 4 * (t->num_scales + 1 + BQ_ABSMAX_CELLS), 512), &t->data,
-                           &t->alloc_bytes);
+  size_t bytes = t->scales_offset + 4 * (t->num_scales + 1 + BQ_ABSMAX_CELLS);
+  if (scheme.tensor_scale) {
+    // two-level: the kernels read global * s_block at scales(); what the blob stores -- the
+    // per-tensor scale, then the block scales -- is kept beside them
+    t->wire_offset = round_up(bytes, 256);
+    bytes = t->wire_offset + 4 * (1 + t->num_scales);
+  }
+  bq_status s = dev->alloc(round_up(bytes, 512), &t->data, &t->alloc_bytes);
   if (s != BQ_OK) {
     delete t;
     return s;
@@ -570,7 +580,8 @@ extern "C" bq_status bq_quantized_data_len(const bq_scheme* scheme, const size_t
   // (a zero block extent, a dim the block does not divide, an unknown store or level are refused
   // here; a ragged last dim is not: the formula pads it to whole words, burn-store's data_len cases)
   BQ_TRY(check_scheme(*scheme, shape, rank, false));
-  *len_out = value_bytes(*scheme, shape, rank) + scale_size(*scheme) * num_params(*scheme, shape, rank);
+  *len_out = value_bytes(*scheme, shape, rank) + scale_size(*scheme) * num_params(*scheme, shape, rank) +
+             global_size(*scheme);
   return BQ_OK;
 }
 
@@ -584,7 +595,7 @@ extern "C" bq_status bq_q_from_data(bq_device* dev, const uint8_t* bytes, size_t
   bq_tensor* t = nullptr;
   BQ_TRY(new_quantized(dev, *scheme, shape, rank, &t));
   const size_t ssz = scale_size(*scheme);
-  const size_t need = t->value_bytes + ssz * t->num_scales;
+  const size_t need = t->value_bytes + ssz * t->num_scales + global_size(*scheme);
   if (len != need) {
     bq_tensor_release(t);
     BQ_FAIL(BQ_ERR_SIZE, "quantized tensor data is %zu bytes, its scheme and shape need %zu", len, need);
@@ -595,7 +606,10 @@ extern "C" bq_status bq_q_from_data(bq_device* dev, const uint8_t* bytes, size_t
   }
   hipError_t e = hipSuccess;
   bq_status rc = BQ_OK;
-  if (ssz == 4 && t->scales_offset == t->value_bytes) {
+  const bool two_level = scheme->tensor_scale != 0;
+  // two-level: the block scales go to the stored copy, the kernels' scales are derived below
+  float* const scales_dst = two_level ? t->wire_scales() : t->scales();
+  if (!two_level && ssz == 4 && t->scales_offset == t->value_bytes) {
     // the device layout is the wire layout (values of a multiple of 256 bytes, f32 scales right
     // behind them): the whole blob arrives with one copy
     e = hipMemcpyAsync(t->data, bytes, need, hipMemcpyHostToDevice, dev->stream);
@@ -609,7 +623,7 @@ extern "C" bq_status bq_q_from_data(bq_device* dev, const uint8_t* bytes, size_t
   }
   if (t->value_bytes) e = hipMemcpyAsync(t->data, bytes, t->value_bytes, hipMemcpyHostToDevice, dev->stream);
   if (e == hipSuccess && ssz == 4) {
-    e = hipMemcpyAsync(t->scales(), bytes + t->value_bytes, 4 * t->num_scales, hipMemcpyHostToDevice, dev->stream);
+    e = hipMemcpyAsync(scales_dst, bytes + t->value_bytes, 4 * t->num_scales, hipMemcpyHostToDevice, dev->stream);
   } else if (e == hipSuccess) {
     // 2-byte scales: staged in a device block, widened (exactly) to the f32 the kernels read
     void* stage = nullptr;
@@ -617,9 +631,13 @@ extern "C" bq_status bq_q_from_data(bq_device* dev, const uint8_t* bytes, size_t
     rc = dev->alloc(2 * t->num_scales, &stage, &stage_bytes);
     if (rc == BQ_OK) {
       e = hipMemcpyAsync(stage, bytes + t->value_bytes, 2 * t->num_scales, hipMemcpyHostToDevice, dev->stream);
-      if (e == hipSuccess) rc = launch_scales_from_wire(stage, t->scales(), t->num_scales, scheme->scale_dtype, dev->stream);
+      if (e == hipSuccess) rc = launch_scales_from_wire(stage, scales_dst, t->num_scales, scheme->scale_dtype, dev->stream);
       dev->release(stage, stage_bytes);  // (stream ordered: the next owner's work queues behind the kernel)
     }
+  }
+  if (two_level && e == hipSuccess && rc == BQ_OK) {
+    e = hipMemcpyAsync(t->wire_global(), bytes + t->value_bytes + ssz * t->num_scales, 4, hipMemcpyHostToDevice, dev->stream);
+    if (e == hipSuccess) rc = launch_scales_times_global(t->wire_scales(), t->wire_global(), t->num_scales, t->scales(), dev->stream);
   }
   if (e == hipSuccess) e = hipStreamSynchronize(dev->stream);
   if (e != hipSuccess || rc != BQ_OK) {
@@ -636,26 +654,30 @@ extern "C" bq_status bq_q_into_data(const bq_tensor* t, uint8_t* bytes, size_t c
   BQ_NOTNULL(len_out);
   if (t->dtype != BQ_QFLOAT) BQ_FAIL(BQ_ERR_DTYPE, "bq_q_into_data on a float tensor");
   const size_t ssz = scale_size(t->scheme);
-  const size_t need = t->value_bytes + ssz * t->num_scales;
+  const size_t need = t->value_bytes + ssz * t->num_scales + global_size(t->scheme);
   *len_out = need;
   if (capacity < need) BQ_FAIL(BQ_ERR_SIZE, "host buffer of %zu bytes for a blob of %zu", capacity, need);
   BQ_NOTNULL(bytes);
   hipStream_t st = t->dev->stream;
-  if (ssz == 4 && t->scales_offset == t->value_bytes) {  // dense on the device as on the wire: one copy
+  const bool two_level = t->scheme.tensor_scale != 0;
+  const float* const scales_src = two_level ? t->wire_scales() : t->scales();
+  if (two_level)  // the per-tensor scale comes last (every path below ends with a synchronisation)
+    BQ_HIP(hipMemcpyAsync(bytes + t->value_bytes + ssz * t->num_scales, t->wire_global(), 4, hipMemcpyDeviceToHost, st));
+  if (!two_level && ssz == 4 && t->scales_offset == t->value_bytes) {  // dense on the device as on the wire: one copy
     BQ_HIP(hipMemcpyAsync(bytes, t->data, need, hipMemcpyDeviceToHost, st));
     BQ_HIP(hipStreamSynchronize(st));
     return BQ_OK;
   }
   if (t->value_bytes) BQ_HIP(hipMemcpyAsync(bytes, t->data, t->value_bytes, hipMemcpyDeviceToHost, st));
   if (ssz == 4) {
-    BQ_HIP(hipMemcpyAsync(bytes + t->value_bytes, t->scales(), 4 * t->num_scales, hipMemcpyDeviceToHost, st));
+    BQ_HIP(hipMemcpyAsync(bytes + t->value_bytes, scales_src, 4 * t->num_scales, hipMemcpyDeviceToHost, st));
     BQ_HIP(hipStreamSynchronize(st));
     return BQ_OK;
   }
   void* stage = nullptr;
   size_t stage_bytes = 0;
   BQ_TRY(t->dev->alloc(2 * t->num_scales, &stage, &stage_bytes));
-  bq_status rc = launch_scales_to_wire(t->scales(), stage, t->num_scales, t->scheme.scale_dtype, st);
+  bq_status rc = launch_scales_to_wire(scales_src, stage, t->num_scales, t->scheme.scale_dtype, st);
   hipError_t e = hipSuccess;
   if (rc == BQ_OK) e = hipMemcpyAsync(bytes + t->value_bytes, stage, 2 * t->num_scales, hipMemcpyDeviceToHost, st);
   if (e == hipSuccess) e = hipStreamSynchronize(st);
@@ -699,14 +721,27 @@ static bq_status validate_quantize_inputs(bq_device* dev, const float* x, size_t
   return BQ_OK;
 }
 
+static bq_status quantize_pass(const bq_tensor* x, const bq_scheme* scheme, bq_tensor* q, const bq_tensor* scales,
+                               const bq_tensor* global, bool dynamic, bool params_ready, int sdt);
+
 static bq_status quantize_impl(const bq_tensor* x, const bq_scheme* scheme, const bq_tensor* scales,
-                               bq_tensor** out) {
+                               bq_tensor** out, const bq_tensor* global = nullptr) {
   BQ_NOTNULL(x);
   BQ_NOTNULL(scheme);
   BQ_NOTNULL(out);
   if (x->dtype != BQ_F32)
     BQ_FAIL(BQ_ERR_DTYPE, "quantize takes an f32 tensor (got dtype %d)", x->dtype);
   const bool dynamic = scales == nullptr;
+  const bool two_level = scheme->tensor_scale != 0;
+  // (the reference's messages: QuantizedBytes::new, crates/burn-std/src/tensor/quantization.rs:259-261)
+  if (!dynamic && two_level && global == nullptr) BQ_FAIL(BQ_ERR_SHAPE, "a two-level scheme requires a per-tensor scale");
+  if (global != nullptr && !two_level) BQ_FAIL(BQ_ERR_SHAPE, "this scheme does not take a per-tensor scale");
+  if (global != nullptr && (global->dtype != BQ_F32 || global->numel() != 1 || global->dev != x->dev))
+    BQ_FAIL(BQ_ERR_SHAPE, "the per-tensor scale must be an f32 tensor of one element on the input's device");
+  // (normalize_scales, crates/burn-backend/src/quantization/scheme.rs:115-118)
+  if (dynamic && two_level && scheme->scale_dtype != BQ_SCALE_F16)
+    BQ_FAIL(BQ_ERR_UNSUPPORTED_SCHEME,
+            "block scales of this dtype reach f32's range, which a per-tensor scale cannot absorb (f16 block scales can)");
   bq_tensor* q = nullptr;
   BQ_TRY(new_quantized(x->dev, *scheme, x->shape, x->rank, &q));
   if (!dynamic) {
@@ -727,9 +762,53 @@ static bq_status quantize_impl(const bq_tensor* x, const bq_scheme* scheme, cons
       return rc;
     }
   }
-  const int sdt = scheme->scale_dtype;
+  // Two-level: the kernels below always see the final f32 scale of a block, global * s_block. Given
+  // parameters are combined first; a dynamic call computes plain f32 block scales in a first pass
+  // over x (the values it writes are overwritten), splits them, and quantizes against the products.
+  const int sdt = two_level ? BQ_SCALE_F32 : scheme->scale_dtype;
+  bool dynamic_pass = dynamic;
+  for (int pass = 0; pass < 2; ++pass) {
+    if (pass == 1) {
+      if (!(two_level && dynamic) || rc != BQ_OK || n == 0) break;
+      uint32_t* cells = reinterpret_cast<uint32_t*>(q->scales() + q->num_scales);
+      rc = bqk_absmax_f32(q->scales(), q->num_scales, cells, st);
+      if (rc == BQ_OK)
+        rc = launch_two_level_split(q->scales(), q->num_scales, cells, scheme->scale_dtype, q->wire_global(), q->wire_scales(), st);
+      if (rc != BQ_OK) break;
+      dynamic_pass = false;
+    }
+    rc = quantize_pass(x, scheme, q, scales, global, dynamic_pass, pass == 1, sdt);
+  }
+  if (rc != BQ_OK) {
+    bq_tensor_release(q);
+    return rc;
+  }
+  *out = q;
+  return BQ_OK;
+}
+
+// One pass of quantize_impl: parameters in place (unless they already are), then the value kernels.
+static bq_status quantize_pass(const bq_tensor* x, const bq_scheme* scheme, bq_tensor* q, const bq_tensor* scales,
+                               const bq_tensor* global, bool dynamic, bool params_ready, int sdt) {
+  hipStream_t st = x->dev->stream;
+  const size_t n = x->numel();
+  const float* xin = static_cast<const float*>(x->data);
+  const bool two_level = scheme->tensor_scale != 0;
+  bq_status rc = BQ_OK;
   do {
-    if (!dynamic) {
+    if (!dynamic && !params_ready && two_level) {
+      // s_block rounded up to the scale dtype, kept as stored; the block's scale is global * that
+      rc = launch_round_scales(static_cast<const float*>(scales->data), q->wire_scales(), q->num_scales, scheme->scale_dtype, st);
+      if (rc != BQ_OK) break;
+      hipError_t e = hipMemcpyAsync(q->wire_global(), global->data, 4, hipMemcpyDeviceToDevice, st);
+      if (e != hipSuccess) {
+        set_error("copying the per-tensor scale failed: %s", hipGetErrorString(e));
+        rc = BQ_ERR_HIP;
+        break;
+      }
+      rc = launch_scales_times_global(q->wire_scales(), q->wire_global(), q->num_scales, q->scales(), st);
+      if (rc != BQ_OK) break;
+    } else if (!dynamic && !params_ready) {
       // the stored scale is the given one, rounded up to the scale dtype first (scale_to_dtype,
       // crates/burn-ndarray/src/ops/qtensor.rs:90-95): the values are divided by what is stored
       if (sdt == BQ_SCALE_F32) {
@@ -781,18 +860,20 @@ static bq_status quantize_impl(const bq_tensor* x, const bq_scheme* scheme, cons
                                 q->data, q->scales(), st);
     }
   } while (false);
-  if (rc != BQ_OK) {
-    bq_tensor_release(q);
-    return rc;
-  }
-  *out = q;
-  return BQ_OK;
+  return rc;
 }
 
 extern "C" bq_status bq_quantize(const bq_tensor* x, const bq_scheme* scheme, const bq_tensor* scales,
                                  bq_tensor** out) {
   BQ_NOTNULL(scales);
   return quantize_impl(x, scheme, scales, out);
+}
+
+extern "C" bq_status bq_quantize_two_level(const bq_tensor* x, const bq_scheme* scheme, const bq_tensor* scales,
+                                           const bq_tensor* global, bq_tensor** out) {
+  BQ_NOTNULL(scales);
+  BQ_NOTNULL(global);
+  return quantize_impl(x, scheme, scales, out, global);
 }
 
 extern "C" bq_status bq_quantize_dynamic(const bq_tensor* x, const bq_scheme* scheme, bq_tensor** out) {
@@ -1144,6 +1225,7 @@ static bq_tensor* alias_of(const bq_tensor* t) {
   a->value_bytes = t->value_bytes;
   a->scales_offset = t->scales_offset;
   a->num_scales = t->num_scales;
+  a->wire_offset = t->wire_offset;
   bq_tensor* root = const_cast<bq_tensor*>(t->base ? t->base : t);
   root->refs.fetch_add(1);
   a->base = root;
@@ -1163,8 +1245,8 @@ extern "C" bq_status bq_q_to_device(const bq_tensor* t, bq_device* dev, bq_tenso
   bq_tensor* q = nullptr;
   BQ_TRY(new_quantized(dev, t->scheme, t->shape, t->rank, &q));
   BQ_HIP(hipStreamSynchronize(t->dev->stream));
-  hipError_t e = hipMemcpyPeerAsync(q->data, dev->ordinal, t->data, t->dev->ordinal,
-                                    t->scales_offset + 4 * t->num_scales, dev->stream);
+  const size_t span = t->scheme.tensor_scale ? t->wire_offset + 4 * (1 + t->num_scales) : t->scales_offset + 4 * t->num_scales;
+  hipError_t e = hipMemcpyPeerAsync(q->data, dev->ordinal, t->data, t->dev->ordinal, span, dev->stream);
   if (e != hipSuccess) {
     bq_tensor_release(q);
     BQ_FAIL(BQ_ERR_HIP, "peer copy failed: %s", hipGetErrorString(e));
@@ -1254,7 +1336,19 @@ static bq_status q_gather_impl(const bq_tensor* t, const int32_t* axes, const ui
   bq_status rc = launch_q_gather(t->data, q->data, t->shape, rank, axes, flip, scheme.value,
                                  scheme.store == BQ_STORE_NATIVE, st);
   if (rc == BQ_OK) {
-    if (scheme.level == BQ_LEVEL_BLOCK && !keep_params) {
+    if (scheme.tensor_scale) {  // two-level: what the blob stores moves like the scales the kernels use
+      hipError_t e = hipMemcpyAsync(q->wire_global(), t->wire_global(), 4, hipMemcpyDeviceToDevice, st);
+      if (e == hipSuccess && keep_params)
+        e = hipMemcpyAsync(q->wire_scales(), t->wire_scales(), 4 * t->num_scales, hipMemcpyDeviceToDevice, st);
+      if (e != hipSuccess) {
+        set_error("copying scales failed: %s", hipGetErrorString(e));
+        rc = BQ_ERR_HIP;
+      } else if (!keep_params) {
+        rc = launch_f32_gather(t->wire_scales(), q->wire_scales(), old_params, rank, axes, flip, st);
+      }
+    }
+    if (rc != BQ_OK) {
+    } else if (scheme.level == BQ_LEVEL_BLOCK && !keep_params) {
       rc = launch_f32_gather(t->scales(), q->scales(), old_params, rank, axes, flip, st);
     } else {
       hipError_t e = hipMemcpyAsync(q->scales(), t->scales(), 4 * t->num_scales, hipMemcpyDeviceToDevice, st);

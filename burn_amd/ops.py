@@ -231,20 +231,28 @@ class TensorData:
         check(lib().bq_quantized_data_len(C.byref(c), sh, rank, C.byref(n)))
         return n.value
 
+    def global_scale(self):
+        """The per-tensor scale of a two-level blob (its last four bytes), else None."""
+        if self.scheme.tensor_scale is None:
+            return None
+        return self.bytes[self.bytes.size - 4:].copy().view(np.float32)[0]
+
     def split(self):
         """(values bytes, scales as f32) -- the two regions of the blob. 2-byte scales (f16 / bf16)
-        are widened exactly (decode_scales, crates/burn-std/src/tensor/quantization.rs:418-441)."""
+        are widened exactly (decode_scales, crates/burn-std/src/tensor/quantization.rs:418-441). A
+        two-level blob ends with its per-tensor scale (`global_scale`), which is not part of them."""
         from .quantization import ScaleDtype
         pshape = params_shape(self.shape, self.scheme)
         n_scales = int(np.prod(pshape))
-        cut = self.bytes.size - self.scheme.scale_dtype.size() * n_scales
-        raw = self.bytes[cut:]
+        end = self.bytes.size - (0 if self.scheme.tensor_scale is None else 4)
+        cut = end - self.scheme.scale_dtype.size() * n_scales
+        raw = self.bytes[cut:end]
         if self.scheme.scale_dtype == ScaleDtype.F32:
-            scales = raw.view(np.float32)
+            scales = raw.copy().view(np.float32)
         elif self.scheme.scale_dtype == ScaleDtype.F16:
-            scales = raw.view(np.float16).astype(np.float32)
+            scales = raw.copy().view(np.float16).astype(np.float32)
         else:
-            scales = f32_from_bf16_bits(raw.view(np.uint16))
+            scales = f32_from_bf16_bits(raw.copy().view(np.uint16))
         return self.bytes[:cut], scales.reshape(pshape)
 
 
@@ -269,10 +277,15 @@ class QTensorOps:
         return TensorData(out[: n.value], t.shape, scheme)
 
     @staticmethod
-    def quantize(tensor: Tensor, scheme: QuantScheme, scales: Tensor) -> Tensor:
+    def quantize(tensor: Tensor, scheme: QuantScheme, scales: Tensor, global_scale: Optional[Tensor] = None) -> Tensor:
+        """quantize(tensor, scheme, qparams): `global_scale` is qparams.global, the one-element f32
+        tensor a two-level scheme takes besides its block scales."""
         c = scheme.to_c()
         h = C.c_void_p()
-        check(lib().bq_quantize(tensor.handle, C.byref(c), scales.handle, C.byref(h)))
+        if global_scale is None:
+            check(lib().bq_quantize(tensor.handle, C.byref(c), scales.handle, C.byref(h)))
+        else:
+            check(lib().bq_quantize_two_level(tensor.handle, C.byref(c), scales.handle, global_scale.handle, C.byref(h)))
         return _wrap(h, tensor.device)
 
     @staticmethod

@@ -2,8 +2,8 @@
 
 `QuantScheme` mirrors cubecl_common::quant::scheme::QuantScheme as burn re-exports it
 (crates/burn-std/src/tensor/quantization.rs:4-6), restricted to what this backend implements:
-symmetric Q8S / Q4S values, per-tensor or per-block scales stored as f32, f16 or bf16, Native or
-PackedU32(0) store.
+symmetric Q8S / Q4S / Q2S values, per-tensor or per-block scales stored as f32, f16 or bf16, an
+optional f32 per-tensor scale on top of block scales (two-level), Native or PackedU32(0) store.
 """
 from __future__ import annotations
 
@@ -43,13 +43,15 @@ class ScaleDtype(IntEnum):
 
 @dataclass(frozen=True)
 class QuantScheme:
-    """value / level (block None = per tensor) / store / scale dtype. `QuantScheme()` is the
-    reference default: Q8S, per-tensor, PackedU32(0), f32 scales."""
+    """value / level (block None = per tensor) / store / scale dtype / per-tensor scale on top of
+    block scales. `QuantScheme()` is the reference default: Q8S, per-tensor, PackedU32(0), f32
+    scales."""
 
     value: QuantValue = QuantValue.Q8S
     block: Optional[Tuple[int, ...]] = None
     store: QuantStore = QuantStore.PackedU32
     scale_dtype: ScaleDtype = ScaleDtype.F32
+    tensor_scale: Optional[ScaleDtype] = None   # block schemes only: two-level (global_scale_dtype)
 
     def with_value(self, value: QuantValue) -> "QuantScheme":
         return replace(self, value=value)
@@ -58,10 +60,25 @@ class QuantScheme:
         return replace(self, store=store)
 
     def per_block(self, block, scale_dtype: ScaleDtype = ScaleDtype.F32) -> "QuantScheme":
-        return replace(self, block=tuple(int(b) for b in block), scale_dtype=scale_dtype)
+        """Block scales of `scale_dtype` (one level: a per-tensor scale on top is dropped)."""
+        return replace(self, block=tuple(int(b) for b in block), scale_dtype=scale_dtype, tensor_scale=None)
 
     def per_tensor(self, scale_dtype: Optional[ScaleDtype] = None) -> "QuantScheme":
-        return replace(self, block=None, scale_dtype=self.scale_dtype if scale_dtype is None else scale_dtype)
+        """A per-tensor scale of `scale_dtype`. On a block scheme it comes on top of the block scales
+        (two-level, as `.per_block(b, dt).per_tensor(ScaleDtype::F32)` in the reference) and has to
+        be f32 ("a two-level scheme stores its per-tensor scale as f32",
+        crates/burn-std/src/tensor/quantization.rs:250-255); otherwise it is the scheme's one scale."""
+        dtype = ScaleDtype.F32 if scale_dtype is None and self.block is not None else scale_dtype
+        if self.block is not None:
+            if dtype != ScaleDtype.F32:
+                raise ValueError("a two-level scheme stores its per-tensor scale as f32")
+            return replace(self, tensor_scale=ScaleDtype.F32)
+        return replace(self, scale_dtype=self.scale_dtype if dtype is None else dtype)
+
+    def per_tensor_only(self, scale_dtype: Optional[ScaleDtype] = None) -> "QuantScheme":
+        """Back to one scale for the whole tensor."""
+        return replace(self, block=None, tensor_scale=None,
+                       scale_dtype=self.scale_dtype if scale_dtype is None else scale_dtype)
 
     def with_scale_dtype(self, scale_dtype: ScaleDtype) -> "QuantScheme":
         return replace(self, scale_dtype=scale_dtype)
@@ -78,6 +95,9 @@ class QuantScheme:
         c.value = int(self.value)
         c.store = int(self.store)
         c.scale_dtype = int(self.scale_dtype)
+        c.tensor_scale = 0 if self.tensor_scale is None else 1
+        if self.tensor_scale is not None and self.block is None:
+            raise ValueError("a per-tensor scale on top goes with block scales")
         if self.block is None:
             c.level = _lib.LEVEL_TENSOR
             c.block_rank = 0
@@ -97,7 +117,8 @@ class QuantScheme:
         block = None
         if c.level == _lib.LEVEL_BLOCK:
             block = tuple(c.block[i] for i in range(c.block_rank))
-        return cls(QuantValue(c.value), block, QuantStore(c.store), ScaleDtype(c.scale_dtype))
+        return cls(QuantValue(c.value), block, QuantStore(c.store), ScaleDtype(c.scale_dtype),
+                   ScaleDtype.F32 if c.tensor_scale else None)
 
 
 def params_shape(shape, scheme: QuantScheme):

@@ -75,9 +75,17 @@ typedef struct bq_scheme {
   uint8_t store;       /* BQ_STORE_NATIVE (Q8S only) | BQ_STORE_PACKED_U32 */
   uint8_t scale_dtype; /* BQ_SCALE_F32 | BQ_SCALE_F16 | BQ_SCALE_BF16 */
   uint8_t block_rank;
-  uint8_t reserved[3];
+  uint8_t tensor_scale; /* block level only: 1 = an f32 per-tensor scale on top of the block scales (below) */
+  uint8_t reserved[2];
   uint8_t block[BQ_MAX_RANK];
 } bq_scheme;
+/* Two-level schemes (`.per_block(b, dtype).per_tensor(ScaleDtype::F32)`; global_scale_dtype,
+ * crates/burn-std/src/tensor/quantization.rs:134-136): the scale of a block is global * s_block, the
+ * block scales are stored in the scale dtype and the per-tensor scale as one f32 behind them
+ * (QuantizedBytes::new, same file :245-266). quantize_dynamic splits the block scales so that the
+ * largest lands on the scale dtype's largest value (normalize_scales,
+ * crates/burn-backend/src/quantization/scheme.rs:106-134), which the reference allows for scale
+ * dtypes whose largest value does not exceed f16's: here that is BQ_SCALE_F16. */
 
 typedef struct bq_device bq_device; /* one GPU: stream, allocation cache, workspace */
 typedef struct bq_tensor bq_tensor; /* ref-counted device tensor: float, or values || scales */
@@ -190,8 +198,15 @@ bq_status bq_q_into_data(const bq_tensor* t, uint8_t* bytes, size_t capacity, si
 /* QTensorOps::quantize (qtensor.rs:137): `scales` is an f32 tensor of params_shape entries.
  * q = clamp(round_half_away(x / (s == 0 ? 0.1 : s)), a, b); the stored scale stays s
  * (burn-ndarray/src/ops/qtensor.rs:82-186, ops/quantization.rs:78-133). */
+/* (A two-level scheme takes its parameters through bq_quantize_two_level.) */
 bq_status bq_quantize(const bq_tensor* x, const bq_scheme* scheme, const bq_tensor* scales,
                       bq_tensor** out);
+/* QTensorOps::quantize with QuantizationParametersPrimitive { scales, global: Some(..) }
+ * (crates/burn-backend/src/quantization/parameters.rs:12-20) for a two-level scheme: `global` is an
+ * f32 tensor of one element; every block is quantized against global * scale_to_dtype(s_block)
+ * (quantize_per_block, crates/burn-ndarray/src/ops/qtensor.rs:519-538). */
+bq_status bq_quantize_two_level(const bq_tensor* x, const bq_scheme* scheme, const bq_tensor* scales,
+                                const bq_tensor* global, bq_tensor** out);
 /* QTensorOps::quantize_dynamic (qtensor.rs:144-149), overridden as one fused pass per block
  * scheme / two passes per tensor: scale = (2 * max|x|) / (b - a)
  * (crates/burn-backend/src/quantization/scheme.rs:44-104), then quantize as above. */

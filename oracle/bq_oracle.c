@@ -520,6 +520,33 @@ float bqo_scale_to_dtype(float scale, int dtype) {
 
 size_t bqo_scale_size(int dtype) { return dtype == BQO_SCALE_F32 ? 4 : 2; }
 
+/* normalize_scales (burn-backend/src/quantization/scheme.rs:106-134): the per-tensor scale of a
+ * two-level scheme is the largest block scale over the block dtype's largest value, kept at or
+ * above the smallest normal f32; every block scale is divided by it. One f32 operation per step,
+ * as the tensor ops there (float_max, float_div_scalar, float_clamp_min, float_div). Returns the
+ * per-tensor scale, or NaN for a block dtype the reference refuses (its largest value must not
+ * exceed f16's: of f32 / f16 / bf16 that leaves f16, largest value 65504). */
+float bqo_normalize_scales(float* scales, size_t n, int block_dtype) {
+  if (block_dtype != BQO_SCALE_F16) return NAN;
+  float top = scales[0];
+  for (size_t i = 1; i < n; ++i) top = scales[i] > top ? scales[i] : top;
+  float global = top / 65504.0f;
+  if (global < 1.17549435e-38f) global = 1.17549435e-38f;   /* f32::MIN_POSITIVE */
+  for (size_t i = 0; i < n; ++i) scales[i] = scales[i] / global;
+  return global;
+}
+
+/* What NdArray::quantize makes of two-level parameters (burn-ndarray/src/ops/qtensor.rs:90-101,
+ * 519-531): the block scales are rounded up to the block dtype (they are stored that way), the
+ * per-tensor scale stays f32, and block i is quantized against global * stored[i]. */
+void bqo_two_level_scales(const float* block_scales, size_t n, int block_dtype, float global, float* stored,
+                          float* effective) {
+  for (size_t i = 0; i < n; ++i) {
+    stored[i] = bqo_scale_to_dtype(block_scales[i], block_dtype);
+    effective[i] = global * stored[i];
+  }
+}
+
 void bqo_encode_scales(const float* scales, size_t n, int dtype, uint8_t* out) {
   for (size_t i = 0; i < n; ++i) {
     if (dtype == BQO_SCALE_F32) {

@@ -41,6 +41,16 @@
  *                        value becomes (this restatement saturates to it, as the reference's test
  *                        comment says of e4m3), and UE4M3 / UE8M0 (not implemented).
  *   bqo_encode/decode_scales  same test (:631-657) and the two-level layout test (:659-684).
+ *   bqo_normalize_scales, bqo_two_level_scales  restated step for step from the reference's tensor
+ *                        ops; no reference-held numbers exist. Pinned by what the mathematics
+ *                        fixes (the largest stored block scale is exactly the dtype's largest
+ *                        value, 65504, unless the clamp acts; global * stored >= the one-level
+ *                        scale, within one f16 step of it) and by the reference's own properties
+ *                        (burn-backend-tests .../ops/quantize.rs:213-293, 489-516: the blob round
+ *                        trip reproduces the dequantized values exactly, they are within 1e-2 of
+ *                        the input, and the error does not track the weights' magnitude). The
+ *                        largest value of the block dtype is f16's by the reference's own assert
+ *                        (scheme.rs:115-118); UE4M3 blocks are not implemented.
  */
 #ifndef BQ_ORACLE_H
 #define BQ_ORACLE_H
@@ -124,6 +134,14 @@ float bqo_scale_to_dtype(float scale, int dtype);
 /* scale_size / encode_scales / decode_scales (same file, :409-464): bytes per scale on the wire;
  * f16 and bf16 are written with round-to-nearest-even (half::from_f32), native endian. */
 size_t bqo_scale_size(int dtype);
+/* Two-level schemes (block scales in a narrow dtype + one f32 per-tensor scale; global_scale_dtype,
+ * burn-std/src/tensor/quantization.rs:134-136). normalize_scales (burn-backend/src/quantization/
+ * scheme.rs:106-134) divides the block scales in place by global = max / dtype_max and returns
+ * global (NaN for a block dtype the reference refuses); two_level_scales gives what is stored and
+ * what a block is quantized against (burn-ndarray/src/ops/qtensor.rs:90-101, 519-531). */
+float bqo_normalize_scales(float* scales, size_t n, int block_dtype);
+void bqo_two_level_scales(const float* block_scales, size_t n, int block_dtype, float global, float* stored,
+                          float* effective);
 void bqo_encode_scales(const float* scales, size_t n, int dtype, uint8_t* out);
 void bqo_decode_scales(const uint8_t* in, size_t n, int dtype, float* out);
 

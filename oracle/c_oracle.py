@@ -48,9 +48,8 @@ class Scheme(C.Structure):
 
 
 def build(force: bool = False) -> str:
-    if force or not os.path.exists(_LIB_PATH):
-        subprocess.run(["make", "-C", _HERE, "-B" if force else "-s"], check=True,
-                       stdout=subprocess.DEVNULL)
+    # (make compares time stamps: a library older than its sources is rebuilt, a current one is not)
+    subprocess.run(["make", "-C", _HERE, "-B" if force else "-s"], check=True, stdout=subprocess.DEVNULL)
     return _LIB_PATH
 
 
@@ -105,6 +104,10 @@ def lib():
         L.bqo_encode_scales.restype = None
         L.bqo_decode_scales.argtypes = [pu8, sz, i32, pf]
         L.bqo_decode_scales.restype = None
+        L.bqo_normalize_scales.argtypes = [pf, sz, i32]
+        L.bqo_normalize_scales.restype = C.c_float
+        L.bqo_two_level_scales.argtypes = [pf, sz, i32, C.c_float, pf, pf]
+        L.bqo_two_level_scales.restype = None
         _lib = L
     return _lib
 
@@ -312,3 +315,45 @@ def ternary_matmul(lhs, rhs_q, gamma):
     out = np.empty((m, n), np.float32)
     lib().bqo_ternary_matmul(_p(lhs, C.c_float), m, k, n, _p(rhs_q, C.c_int8), float(gamma), _p(out, C.c_float))
     return out
+
+
+# ---- two-level schemes: block scales in a narrow dtype + one f32 per-tensor scale -------------------
+
+def normalize_scales(scales, block_dtype):
+    """normalize_scales (burn-backend/src/quantization/scheme.rs:106-134) -> (relative block scales, global)."""
+    a = np.ascontiguousarray(scales, dtype=np.float32).copy()
+    g = lib().bqo_normalize_scales(_p(a.reshape(-1), C.c_float), a.size, block_dtype)
+    if g != g:
+        raise ValueError("block scales of this dtype reach f32's range, which a per-tensor scale cannot absorb")
+    return a, np.float32(g)
+
+
+def two_level_scales(block_scales, block_dtype, global_scale):
+    """(stored block scales, scale each block is quantized against = global * stored)."""
+    a = np.ascontiguousarray(block_scales, dtype=np.float32)
+    stored, eff = np.empty_like(a), np.empty_like(a)
+    lib().bqo_two_level_scales(_p(a.reshape(-1), C.c_float), a.size, block_dtype, float(global_scale),
+                               _p(stored.reshape(-1), C.c_float), _p(eff.reshape(-1), C.c_float))
+    return stored, eff
+
+
+def quantize_two_level(x, scheme, block_scales, global_scale, block_dtype):
+    """NdArray::quantize with QuantizationParametersPrimitive { scales, global: Some(..) }:
+    -> (values, stored block scales, effective scales)."""
+    stored, eff = two_level_scales(block_scales, block_dtype, global_scale)
+    return quantize(x, scheme, eff), stored, eff
+
+
+def quantize_dynamic_two_level(x, scheme, block_dtype):
+    """quantize_dynamic of a two-level scheme: range -> one-level f32 block scales -> normalize_scales
+    -> quantize. -> (values, stored block scales, global, effective scales)."""
+    _, scales = quantize_dynamic(x, scheme)
+    rel, g = normalize_scales(scales, block_dtype)
+    q, stored, eff = quantize_two_level(x, scheme, rel, g, block_dtype)
+    return q, stored, g, eff
+
+
+def encode_two_level(q, scheme, stored, global_scale, block_dtype):
+    """QuantizedBytes::new for a two-level scheme: values || block scales in their dtype || f32 global."""
+    blob = encode_with_scale_dtype(q, scheme, stored, block_dtype)
+    return np.concatenate([blob, np.float32([global_scale]).view(np.uint8)])

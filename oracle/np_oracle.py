@@ -185,6 +185,23 @@ def scale_to_dtype(scales, dtype="F32"):
     raise ValueError(dtype)
 
 
+def quantize_dynamic_two_level(x, value="Q8S", block=None, block_dtype="F16"):
+    """quantize_dynamic under a two-level scheme, a second restatement in numpy f32 arithmetic:
+    compute_q_params + normalize_scales (crates/burn-backend/src/quantization/scheme.rs:75-134), then
+    NdArray::quantize against global * scale_to_dtype(relative block scale)
+    (crates/burn-ndarray/src/ops/qtensor.rs:90-101, 519-531).
+    -> (values, stored block scales, global, effective scales)."""
+    if block_dtype != "F16":
+        raise ValueError("block scales of this dtype reach f32's range, which a per-tensor scale cannot absorb")
+    lo, hi = compute_range(x, block)
+    scales = compute_q_params(lo, hi, value).astype(np.float32)
+    g = np.maximum(np.float32(scales.max()) / np.float32(65504.0), np.float32(1.17549435e-38)).astype(np.float32)
+    rel = (scales / g).astype(np.float32)
+    stored = scale_to_dtype(rel, block_dtype)
+    eff = (g * stored).astype(np.float32)
+    return quantize(x, eff, value, block), stored, np.float32(g), eff
+
+
 def ternary_matmul(lhs, q, gamma):
     """crates/burn-ndarray/src/ops/qtensor.rs:431-517: +1 adds, -1 subtracts, anything else is
     skipped, in ascending k; the per-tensor scale multiplies the finished sums."""

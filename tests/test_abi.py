@@ -10,7 +10,7 @@ import pytest
 
 import burn_amd as ba
 from burn_amd import _lib
-from burn_amd.quantization import QuantScheme, QuantStore, QuantValue, params_shape
+from burn_amd.quantization import QuantScheme, QuantStore, QuantValue, ScaleDtype, params_shape
 
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 
@@ -38,6 +38,10 @@ def test_scheme_struct_layout_matches_header():
     assert raw[0] == _lib.Q4S and raw[1] == _lib.LEVEL_BLOCK and raw[2] == _lib.STORE_PACKED_U32
     assert raw[4] == 1 and raw[8] == 32
     assert QuantScheme.from_c(c) == QuantScheme(QuantValue.Q4S, (32,), QuantStore.PackedU32)
+    two = QuantScheme().per_block((2, 16), ScaleDtype.F16).per_tensor(ScaleDtype.F32)
+    raw = bytes(two.to_c())
+    assert raw[3] == _lib.SCALE_F16 and raw[4] == 2 and raw[5] == 1 and raw[8:10] == bytes([2, 16])
+    assert QuantScheme.from_c(two.to_c()) == two and two.per_block((2, 16), ScaleDtype.F16).tensor_scale is None
 
 
 def test_data_len_matches_reference_formula(kats):
@@ -48,6 +52,10 @@ def test_data_len_matches_reference_formula(kats):
     assert ba.TensorData.data_len((16,), QuantScheme().per_block((8,))) == 16 + 8
     assert ba.TensorData.data_len((8192, 8192), QuantScheme().per_block((32,))) == 8192 * 8192 + 4 * 8192 * 256
     assert params_shape((8192, 8192), QuantScheme().per_block((32,))) == (8192, 256)
+    # two-level: block scales in their dtype, then the f32 per-tensor scale
+    # (crates/burn-std/src/tensor/quantization.rs:659-684: 8 values + 2 one-byte scales + 4 there)
+    two = QuantScheme(store=QuantStore.Native).per_block((4,), ScaleDtype.F16).per_tensor()
+    assert ba.TensorData.data_len((8,), two) == 8 + 2 * 2 + 4
     assert params_shape((4, 8), QuantScheme().per_block((2, 4))) == (2, 2)
 
 
@@ -102,6 +110,9 @@ def test_data_len_refuses_what_q_from_data_would_refuse():
     assert status(bad, (4, 64)) == _lib.ERR_UNSUPPORTED_SCHEME
     bad = QuantScheme().to_c()
     bad.level = 5
+    assert status(bad, (4, 64)) == _lib.ERR_UNSUPPORTED_SCHEME
+    bad = QuantScheme().to_c()
+    bad.tensor_scale = 1                                   # a per-tensor scale on top of ... a per-tensor scale
     assert status(bad, (4, 64)) == _lib.ERR_UNSUPPORTED_SCHEME
 
 

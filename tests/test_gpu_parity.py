@@ -745,6 +745,107 @@ def test_q_matmul_with_two_byte_scales(dev, sdt):
 
 # ------------------------------------------------------------------ Q2S ternary weights
 
+# ------------------------------------------------------------------ two-level schemes
+
+def two_level_parts(blob: TensorData):
+    values, stored = blob.split()
+    q = values.view(np.int8).reshape(blob.shape) if blob.scheme.store == QuantStore.Native else \
+        no.unpack_u32(values.view(np.uint32), blob.shape, VAL[blob.scheme.value][1])
+    return q, stored, blob.global_scale()
+
+
+@pytest.mark.parametrize("value,store", [(QuantValue.Q8S, QuantStore.Native), (QuantValue.Q8S, QuantStore.PackedU32),
+                                         (QuantValue.Q4S, QuantStore.PackedU32)])
+@pytest.mark.parametrize("shape,block,mag", [((16, 16), (2, 16), 1.0), ((64, 256), (32,), 0.02), ((4, 6, 32), (1, 2, 16), 300.0),
+                                             ((128, 512), (64,), 1e-6), ((8, 64), (8,), 5.0)])
+def test_two_level_quantize_dynamic(dev, value, store, shape, block, mag):
+    """f16 block scales under an f32 per-tensor scale (`.per_block(b, F16).per_tensor(F32)`): values,
+    stored block scales, the per-tensor scale, the blob and the dequantized floats, all bit for bit
+    against the oracle; and the blob read back gives the same tensor (the reference's round trip,
+    crates/burn-backend-tests/tests/tensor/float/quantization/ops/quantize.rs:489-516)."""
+    x = (np.random.default_rng(len(shape) * 100 + shape[-1]).standard_normal(shape) * mag).astype(np.float32)
+    scheme = QuantScheme(value=value, store=store).per_block(block, ScaleDtype.F16).per_tensor(ScaleDtype.F32)
+    assert scheme.tensor_scale == ScaleDtype.F32 and scheme.block == block
+    osch = oscheme(scheme)
+    q_ref, stored_ref, g_ref, eff_ref = co.quantize_dynamic_two_level(x, osch, co.SCALE_F16)
+    tq = QTensorOps.quantize_dynamic(FloatOps.float_from_data(x, dev), scheme)
+    assert tq.scheme == scheme
+    blob = QTensorOps.q_into_data(tq)
+    q, stored, g = two_level_parts(blob)
+    assert g == g_ref and stored.tobytes() == stored_ref.tobytes() and (q == q_ref).all()
+    assert blob.bytes.tobytes() == co.encode_two_level(q_ref, osch, stored_ref, g_ref, co.SCALE_F16).tobytes()
+    assert blob.bytes.size == TensorData.data_len(shape, scheme)
+    d_ref = co.dequantize(q_ref, osch, eff_ref)
+    assert FloatOps.float_into_data(QTensorOps.dequantize(tq)).tobytes() == d_ref.tobytes()
+    again = QTensorOps.q_from_data(blob, dev)
+    assert FloatOps.float_into_data(QTensorOps.dequantize(again)).tobytes() == d_ref.tobytes()
+    assert QTensorOps.q_into_data(again).bytes.tobytes() == blob.bytes.tobytes()
+
+
+def test_two_level_quantize_with_given_parameters_and_other_ops(dev, tmp_path):
+    rng = np.random.default_rng(77)
+    x = rng.standard_normal((32, 128)).astype(np.float32)
+    block_scales = (np.abs(rng.standard_normal((32, 4))) * 50 + 1).astype(np.float32)   # relative block scales
+    g = np.float32(3.0e-4)
+    for sdt, odt in ((ScaleDtype.F16, co.SCALE_F16), (ScaleDtype.BF16, co.SCALE_BF16), (ScaleDtype.F32, co.SCALE_F32)):
+        scheme = QuantScheme().per_block((32,), sdt).per_tensor(ScaleDtype.F32)
+        q_ref, stored_ref, eff_ref = co.quantize_two_level(x, oscheme(scheme), block_scales, g, odt)
+        tq = QTensorOps.quantize(FloatOps.float_from_data(x, dev), scheme, FloatOps.float_from_data(block_scales, dev),
+                                 FloatOps.float_from_data(np.float32([g]), dev))
+        blob = QTensorOps.q_into_data(tq)
+        q, stored, g_out = two_level_parts(blob)
+        assert g_out == g and stored.tobytes() == stored_ref.tobytes() and (q == q_ref).all()
+        d_ref = co.dequantize(q_ref, oscheme(scheme), eff_ref)
+        assert FloatOps.float_into_data(QTensorOps.dequantize(tq)).tobytes() == d_ref.tobytes()
+    # the products read global * s_block like any other block scale
+    scheme = QuantScheme().per_block((32,), ScaleDtype.F16).per_tensor(ScaleDtype.F32)
+    w = (rng.standard_normal((256, 512)) * 0.03).astype(np.float32)
+    tw = QTensorOps.quantize_dynamic(FloatOps.float_from_data(w, dev), scheme)
+    q_ref, stored_ref, g_ref, eff_ref = co.quantize_dynamic_two_level(w, oscheme(scheme), co.SCALE_F16)
+    wd = co.dequantize(q_ref, oscheme(scheme), eff_ref).astype(np.float64)
+    for m in (1, 8, 64):
+        a = rng.standard_normal((m, 256)).astype(np.float32)
+        out = FloatOps.float_into_data(QTensorOps.q_matmul(FloatOps.float_from_data(a, dev), tw))
+        assert np.abs(out - a.astype(np.float64) @ wd).max() <= (2e-5 if m <= 32 else 1e-2) * np.abs(a.astype(np.float64) @ wd).max()
+    # layout ops carry both sets of parameters; a reshape shares them
+    r = QTensorOps.q_reshape(tw, (128, 1024))
+    assert FloatOps.float_into_data(QTensorOps.dequantize(r)).tobytes() == wd.astype(np.float32).reshape(128, 1024).tobytes()
+    assert QTensorOps.q_into_data(r).bytes.tobytes() == QTensorOps.q_into_data(tw).bytes.tobytes()
+    small = QuantScheme(store=QuantStore.Native).per_block((2, 16), ScaleDtype.F16).per_tensor()
+    xs = rng.standard_normal((8, 32)).astype(np.float32)
+    ts = QTensorOps.quantize_dynamic(FloatOps.float_from_data(xs, dev), small)
+    qs, stored_s, gs, eff_s = co.quantize_dynamic_two_level(xs, oscheme(small), co.SCALE_F16)
+    tt = QTensorOps.q_swap_dims(ts, 0, 1)
+    assert tt.scheme.block == (16, 2) and tt.scheme.tensor_scale == ScaleDtype.F32
+    assert FloatOps.float_into_data(QTensorOps.dequantize(tt)).tobytes() == \
+        co.dequantize(qs, oscheme(small), eff_s).T.copy().tobytes()
+    qt, stored_t, g_t = two_level_parts(QTensorOps.q_into_data(tt))
+    assert g_t == gs and stored_t.tobytes() == stored_s.T.copy().tobytes() and (qt == qs.T).all()
+    tf = QTensorOps.q_flip(ts, [1])
+    qf, stored_f, g_f = two_level_parts(QTensorOps.q_into_data(tf))
+    assert g_f == gs and stored_f.tobytes() == stored_s.tobytes() and (qf == qs[:, ::-1]).all()
+    # burnpack: the scheme travels with the entry
+    path = tmp_path / "two_level.bpk"
+    ba.PackWriter().add_tensor("w", tw).write_to_file(path)
+    reader = ba.PackReader(path)
+    assert reader.find("w")["scheme"] == scheme
+    back = reader.load("w", dev)
+    reader.close()
+    assert back.scheme == scheme
+    assert QTensorOps.q_into_data(back).bytes.tobytes() == QTensorOps.q_into_data(tw).bytes.tobytes()
+    # what the reference refuses
+    bad = QuantScheme().per_block((32,), ScaleDtype.BF16).per_tensor()
+    with pytest.raises(ba.BurnqError):      # normalize_scales: "reach f32's range"
+        QTensorOps.quantize_dynamic(FloatOps.float_from_data(x, dev), bad)
+    with pytest.raises(ba.BurnqError):      # "requires a per-tensor scale"
+        QTensorOps.quantize(FloatOps.float_from_data(x, dev), scheme, FloatOps.float_from_data(block_scales, dev))
+    with pytest.raises(ba.BurnqError):      # "does not take a per-tensor scale"
+        QTensorOps.quantize(FloatOps.float_from_data(x, dev), QuantScheme().per_block((32,)),
+                            FloatOps.float_from_data(block_scales, dev), FloatOps.float_from_data(np.float32([g]), dev))
+    with pytest.raises(ValueError):         # "stores its per-tensor scale as f32"
+        QuantScheme().per_block((32,), ScaleDtype.F16).per_tensor(ScaleDtype.F16)
+
+
 @pytest.mark.parametrize("block", [None, (16,), (32,), (2, 32)])
 def test_q2s_quantize_dequantize(dev, block):
     x = awkward((32, 96), 33)

@@ -413,3 +413,76 @@ def test_ternary_matmul_as_the_reference_checks_it():
     word = co.pack_u32(vals, co.Q2S)
     assert word.reshape(-1)[0] == sum(((v & 3) << (2 * i)) for i, v in enumerate([1, -1, 0, 1] * 4))
     assert (co.unpack_u32(word, (1, 16), co.Q2S) == vals).all()
+
+
+# ------------------------------------------------------------------ two-level schemes
+
+def test_two_level_blob_layout_as_the_reference_pins_it():
+    """crates/burn-std/src/tensor/quantization.rs:659-684 with f16 block scales in place of ue4m3
+    (not implemented): exactly representable parameters pin the layout -- values, the block scales in
+    their dtype, the per-tensor f32 scale last, nothing padded between them."""
+    values = np.int8([0, 25, 51, 76, 102, 127, -128, -1])
+    sch = co.Scheme.make(co.Q8S, [4], co.STORE_NATIVE)
+    blob = co.encode_two_level(values, sch, np.float32([0.5, 0.125]), np.float32(3.0), co.SCALE_F16)
+    assert blob.size == 8 + 2 * 2 + 4
+    assert blob[:8].view(np.int8).tolist() == values.tolist()
+    assert blob[8:12].view(np.uint16).tolist() == [0x3800, 0x3000]
+    assert blob[12:].view(np.float32)[0] == np.float32(3.0)
+
+
+def test_two_level_parameters():
+    """normalize_scales + NdArray::quantize, pinned by what the arithmetic fixes: the largest stored
+    block scale is the block dtype's largest value (the division by global = max / 65504 lands it
+    there, and rounding up cannot pass it), every block is quantized against a scale no smaller than
+    its one-level scale and at most one f16 step (2^-10) above it, and the C and numpy restatements
+    agree bit for bit."""
+    rng = np.random.default_rng(21)
+    for shape, block, mag in (((16, 16), [2, 16], 1.0), ((8, 64), [32], 0.02), ((4, 6, 32), [1, 2, 16], 300.0),
+                              ((32, 32), [4, 8], 1e-6)):
+        x = (rng.standard_normal(shape) * mag).astype(np.float32)
+        sch = co.Scheme.make(co.Q8S, block, co.STORE_NATIVE)
+        q, stored, g, eff = co.quantize_dynamic_two_level(x, sch, co.SCALE_F16)
+        qn, stored_n, gn, eff_n = no.quantize_dynamic_two_level(x, "Q8S", block, "F16")
+        assert (q == qn).all() and stored.tobytes() == stored_n.reshape(stored.shape).tobytes()
+        assert g == gn and eff.tobytes() == eff_n.reshape(eff.shape).tobytes()
+        assert stored.max() == np.float32(65504.0)
+        assert (stored == co.scale_to_dtype(stored, co.SCALE_F16)).all()          # stored values are f16 values
+        _, one_level = co.quantize_dynamic(x, sch)
+        assert (eff.astype(np.float64) >= one_level.astype(np.float64) * (1 - 2.0 ** -22)).all()
+        assert (eff.astype(np.float64) <= one_level.astype(np.float64) * (1 + 2.0 ** -10 + 2.0 ** -21)).all()
+        # and the values are the quantization against those scales
+        assert (q == co.quantize(x, sch, eff)).all()
+    with pytest.raises(ValueError):
+        co.normalize_scales(np.float32([1.0, 2.0]), co.SCALE_BF16)   # reaches f32's range (scheme.rs:115-118)
+    with pytest.raises(ValueError):
+        co.normalize_scales(np.float32([1.0, 2.0]), co.SCALE_F32)
+    # an all-zero tensor: global is clamped to the smallest normal f32, the block scales are 0
+    z = np.zeros((4, 32), np.float32)
+    q, stored, g, eff = co.quantize_dynamic_two_level(z, co.Scheme.make(co.Q8S, [32], co.STORE_NATIVE), co.SCALE_F16)
+    assert g == np.float32(1.17549435e-38) and (stored == 0).all() and (q == 0).all()
+
+
+def test_two_level_properties_the_reference_asserts():
+    """crates/burn-backend-tests/tests/tensor/float/quantization/ops/quantize.rs:489-516 (f16 block
+    scales under an f32 per-tensor scale: dequantized within rel 1e-2 / abs 1e-2 of the input, the
+    blob reproduces the values and parameters) and :238-293 (the error does not track the weights'
+    magnitude), on their inputs."""
+    x = (np.arange(256, dtype=np.float32) / np.float32(256)).reshape(16, 16)
+    sch = co.Scheme.make(co.Q8S, [2, 16], co.STORE_NATIVE)
+    q, stored, g, eff = co.quantize_dynamic_two_level(x, sch, co.SCALE_F16)
+    d = co.dequantize(q, sch, eff)
+    assert burn_approx_eq(d, x, 1e-2, 1e-2).all()
+    blob = co.encode_two_level(q, sch, stored, g, co.SCALE_F16)
+    assert blob.size == 256 + 2 * 8 + 4
+    back = co.decode_scales(blob[256:256 + 16], co.SCALE_F16)
+    assert back.tobytes() == stored.reshape(-1).tobytes() and blob[-4:].view(np.float32)[0] == g
+    assert co.dequantize(blob[:256].view(np.int8).reshape(16, 16), sch, (g * back).astype(np.float32)).tobytes() == d.tobytes()
+
+    big = (np.arange(-128, 128, dtype=np.float32) / np.float32(128)).reshape(16, 16)
+    small = (big * np.float32(0.02)).astype(np.float32)
+
+    def error(t):
+        q, _, _, eff = co.quantize_dynamic_two_level(t, sch, co.SCALE_F16)
+        return np.abs(t - co.dequantize(q, sch, eff)).sum() / np.abs(t).sum()
+
+    assert abs(error(small) - error(big)) / error(big) < 0.2
