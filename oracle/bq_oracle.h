@@ -50,7 +50,13 @@
  *                        trip reproduces the dequantized values exactly, they are within 1e-2 of
  *                        the input, and the error does not track the weights' magnitude). The
  *                        largest value of the block dtype is f16's by the reference's own assert
- *                        (scheme.rs:115-118); UE4M3 blocks are not implemented.
+ *                        (scheme.rs:115-118); UE4M3 blocks are not implemented. The quotient
+ *                        top / (top / 65504) is 65504 or one f32 step above it, so this path takes
+ *                        the saturating branch of bqo_scale_to_dtype about half of the time (PARITY
+ *                        UNPINNED, see there). The reference's own two-level tests (ue4m3, same
+ *                        arithmetic against 448) only pass if that branch saturates: on their input
+ *                        arange(-128..128)/128 the quotient is one step above the dtype's top, and an
+ *                        infinite block scale would quantize everything to zero.
  */
 #ifndef BQ_ORACLE_H
 #define BQ_ORACLE_H

@@ -782,6 +782,29 @@ def test_two_level_quantize_dynamic(dev, value, store, shape, block, mag):
     assert QTensorOps.q_into_data(again).bytes.tobytes() == blob.bytes.tobytes()
 
 
+def test_two_level_reference_cases(dev, approx):
+    """The reference's own two-level cases with f16 block scales, on their inputs:
+    crates/burn-backend-tests/tests/tensor/float/quantization/ops/quantize.rs:489-516 (round trip
+    through the blob exact, dequantized within rel 1e-2 / abs 1e-2 of the input) and
+    ops/matmul.rs:253-281 (lhs x quantized within rel 1e-2 of lhs x dequantized)."""
+    x = (np.arange(256, dtype=np.float32) / np.float32(256)).reshape(16, 16)
+    scheme = QuantScheme(store=QuantStore.Native).per_block((2, 16), ScaleDtype.F16).per_tensor(ScaleDtype.F32)
+    tq = QTensorOps.quantize_dynamic(FloatOps.float_from_data(x, dev), scheme)
+    direct = FloatOps.float_into_data(QTensorOps.dequantize(tq))
+    reloaded = QTensorOps.q_from_data(QTensorOps.q_into_data(tq), dev)
+    assert FloatOps.float_into_data(QTensorOps.dequantize(reloaded)).tobytes() == direct.tobytes()
+    approx(direct, x, 1e-2, 1e-2)
+    expected = x.astype(np.float64) @ direct.astype(np.float64)
+    actual = FloatOps.float_into_data(QTensorOps.q_matmul(FloatOps.float_from_data(x, dev), tq))
+    approx(actual, expected, 1e-2, 0)
+    # (the input whose largest relative scale lands one f32 step above 65504 before it is stored)
+    big = (np.arange(-128, 128, dtype=np.float32) / np.float32(128)).reshape(16, 16)
+    tb = QTensorOps.quantize_dynamic(FloatOps.float_from_data(big, dev), scheme)
+    q_ref, stored_ref, g_ref, eff_ref = co.quantize_dynamic_two_level(big, oscheme(scheme), co.SCALE_F16)
+    q, stored, g = two_level_parts(QTensorOps.q_into_data(tb))
+    assert stored.max() == np.float32(65504.0) and g == g_ref and stored.tobytes() == stored_ref.tobytes() and (q == q_ref).all()
+
+
 def test_two_level_quantize_with_given_parameters_and_other_ops(dev, tmp_path):
     rng = np.random.default_rng(77)
     x = rng.standard_normal((32, 128)).astype(np.float32)

@@ -452,6 +452,19 @@ def test_two_level_parameters():
         assert (eff.astype(np.float64) <= one_level.astype(np.float64) * (1 + 2.0 ** -10 + 2.0 ** -21)).all()
         # and the values are the quantization against those scales
         assert (q == co.quantize(x, sch, eff)).all()
+    # the reference's own case (crates/burn-backend-tests/tests/tensor/float/quantization/scheme.rs:50-90,
+    # with f16's largest value where it has ue4m3's 448): the largest relative scale sits on the
+    # dtype's top, and relative scale x global gives the one-level scales back
+    lo, hi = np.float32([-1.8, -0.5, 0.01, -0.04]), np.float32([0.5, 1.8, 0.04, -0.01])
+    one_level = co.compute_q_params(lo, hi, co.Q8S)
+    rel, g = co.normalize_scales(one_level, co.SCALE_F16)
+    # (top / (top / 65504) is 65504 or one f32 step above it; stored, it is 65504: rounding up into
+    # f16 saturates there -- the one branch of scale_to_dtype no reference-held vector fixes)
+    assert np.float32(65504.0) <= rel.max() <= np.nextafter(np.float32(65504.0), np.float32(np.inf))
+    assert co.scale_to_dtype(rel, co.SCALE_F16).max() == np.float32(65504.0)
+    assert burn_approx_eq(rel * g, one_level, 0.005, 1e-5).all()          # Tolerance::default()
+    rel0, g0 = co.normalize_scales(np.zeros(1, np.float32), co.SCALE_F16)  # scheme.rs:92-123
+    assert g0 > 0 and np.isfinite(rel0).all()
     with pytest.raises(ValueError):
         co.normalize_scales(np.float32([1.0, 2.0]), co.SCALE_BF16)   # reaches f32's range (scheme.rs:115-118)
     with pytest.raises(ValueError):
