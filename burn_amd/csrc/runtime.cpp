@@ -1330,6 +1330,12 @@ static bq_status q_gather_impl(const bq_tensor* t, const int32_t* axes, const ui
     scheme.block_rank = static_cast<uint8_t>(rank);
     for (int a = 0; a < rank; ++a) scheme.block[a] = static_cast<uint8_t>(old_blk[axes[a]]);
   }
+  // Q8S words are the same bytes as native values, so a result whose last dim no longer fills whole
+  // words is stored natively instead of being refused (the reference's CPU backend keeps one i8 per
+  // value whatever the store says and permutes freely: ops/quantize.rs:406-431 of its tests ends
+  // with a last dim of 2). Sub-byte values have no native store: those results are refused.
+  if (scheme.store == BQ_STORE_PACKED_U32 && scheme.value == BQ_Q8S && new_shape[rank - 1] % 4 != 0)
+    scheme.store = BQ_STORE_NATIVE;
   bq_tensor* q = nullptr;
   BQ_TRY(new_quantized(t->dev, scheme, new_shape, rank, &q));  // also: "Can't store in u32" for the new last dim
   hipStream_t st = t->dev->stream;

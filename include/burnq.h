@@ -247,7 +247,8 @@ bq_status bq_q_reshape(const bq_tensor* t, const size_t* shape, int32_t rank, bq
  * scales move with their blocks (burn-ndarray/src/ops/qtensor.rs:300-347). The result is a new
  * dense tensor (the block of the scheme is permuted with the axes, so a [1, 32] block becomes
  * [32, 1] under a transpose). An axis out of bounds or repeated, which the reference panics on,
- * returns BQ_ERR_SHAPE, as does a packed result whose last dim is not a whole number of words.
+ * returns BQ_ERR_SHAPE, as does a packed sub-byte result whose last dim is not a whole number of
+ * words (a Q8S result of that kind is stored natively: same bytes, one per value).
  * q_flip flips the values and keeps every parameter where it is, block scales included, as the
  * reference does (burn-ndarray/src/ops/qtensor.rs:338-347): a value flipped into another block
  * is dequantized with that block's scale. */

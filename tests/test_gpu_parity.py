@@ -154,6 +154,71 @@ def test_kat_matmuls(dev, kats, approx):
     approx(FloatOps.float_into_data(out), k["expected"], k["tolerance"]["rel"], 0)
 
 
+def test_reference_matmul_cases_both_operands_quantized(dev, approx):
+    """crates/burn-backend-tests/tests/tensor/float/quantization/ops/matmul.rs:9-139: products of two
+    quantized tensors (`QTensor::int8` = quantize_dynamic, default scheme) against the listed results,
+    relative 2e-2 as there. The reference ignores most of them because their last dims do not fill
+    packed words; with the Native store they run: vectors, 2-D, 3-D, broadcast batches."""
+    native = QuantScheme(store=QuantStore.Native)
+
+    def q(values):
+        return QTensorOps.quantize_dynamic(FloatOps.float_from_data(np.float32(values), dev), native)
+
+    def check(a, b, expected):
+        out = QTensorOps.q_matmul(q(a), q(b))
+        assert out.dtype == ba.F32 and out.shape == np.float32(expected).shape
+        approx(FloatOps.float_into_data(out), np.float32(expected), 2e-2, 0)
+
+    check([[1.0, 2.0, 3.0, 6.35]], [[12.7], [4.0], [5.0], [1.0]], [[42.05]])
+    check([[1.0, 6.35], [2.0, 3.0], [1.0, 3.0]], [[4.0, 8.0, 12.7], [2.0, 3.0, 6.0]],
+          [[16.7, 27.05, 50.8], [14., 25., 43.4], [10., 17., 30.7]])
+    check([[[1.0, 6.35], [2.0, 3.0]]], [[[12.7, 4.0], [2.0, 3.0]]], [[[25.4, 23.05], [31.4, 17.0]]])
+    check([[[[1.0, 7.0], [2.0, 3.0]]], [[[2.0, 5.0], [6.0, 3.0]]]], [[[[9.0, 8.0], [1.0, 4.0]], [[2.0, 7.0], [3.0, 5.0]]]],
+          [[[[16.0, 36.0], [21.0, 28.0]], [[23.0, 42.0], [13.0, 29.0]]],
+           [[[23.0, 36.0], [57.0, 60.0]], [[19.0, 39.0], [21.0, 57.0]]]])
+    check([[[1.0, 7.0], [2.0, 3.0]]], [[[4.0, 7.0], [2.0, 3.0]], [[2.0, 5.0], [6.0, 3.0]]],
+          [[[18.0, 28.0], [14.0, 23.0]], [[44.0, 26.0], [22.0, 19.0]]])
+    with pytest.raises(ba.BurnqError):   # should_panic_when_inner_dimensions_are_not_equal
+        QTensorOps.q_matmul(q([[3., 3.], [4., 4.], [5., 5.], [6., 6.]]), q([[1., 2., 3., 4.]] * 3))
+
+
+def test_reference_transposed_and_permuted_cases(dev, approx):
+    """crates/burn-backend-tests/tests/tensor/float/quantization/ops/quantize.rs:119-169 and 292-488:
+    quantize_dynamic -> dequantize of arange grids, per tensor and per block, directly, on transposed
+    inputs, and with the quantized tensor transposed / permuted before it is dequantized (packed
+    words then straddle blocks: blocks of [1, 2, 16] become [16, 1, 2] under permute([2, 0, 1])).
+    Tolerance::absolute(1e-1).set_relative(1e-2), as there. (Float transposes are host-side: float
+    tensor ops are outside this library.)"""
+    def grid(n, shape):
+        return (np.arange(n, dtype=np.float32) / np.float32(n)).reshape(shape)
+
+    def roundtrip(x, scheme):
+        return FloatOps.float_into_data(QTensorOps.dequantize(QTensorOps.quantize_dynamic(FloatOps.float_from_data(x, dev), scheme)))
+
+    per_tensor = QuantScheme()
+    approx(roundtrip(grid(256, (16, 16)), per_tensor), grid(256, (16, 16)), 1e-2, 1e-1)
+    approx(roundtrip(grid(256, (16, 16)), per_tensor.per_block((2, 16))), grid(256, (16, 16)), 1e-2, 1e-1)
+    # should_quantize_transposed: quantize the transposed input, transpose the result back
+    for n, shape, scheme in ((256, (8, 32), per_tensor), (3072, (48, 64), per_tensor), (2048, (32, 64), per_tensor.per_block((32,)))):
+        x = grid(n, shape)
+        approx(roundtrip(np.ascontiguousarray(x.T), scheme).T, x, 1e-2, 1e-1)
+    # should_dequantize_transposed: transpose the quantized tensor
+    for n, shape, scheme in ((256, (8, 32), per_tensor), (2048, (32, 64), per_tensor.per_block((32,)))):
+        x = grid(n, shape)
+        tq = QTensorOps.quantize_dynamic(FloatOps.float_from_data(x, dev), scheme)
+        d = FloatOps.float_into_data(QTensorOps.dequantize(QTensorOps.q_swap_dims(tq, 0, 1)))
+        approx(d.T, x, 1e-2, 1e-1)
+    # permutes of a [2, 8, 16] tensor in [1, 2, 16] blocks
+    x = grid(256, (2, 8, 16))
+    tq = QTensorOps.quantize_dynamic(FloatOps.float_from_data(x, dev), per_tensor.per_block((1, 2, 16)))
+    for axes in ((1, 2, 0), (2, 0, 1)):
+        d = FloatOps.float_into_data(QTensorOps.dequantize(QTensorOps.q_permute(tq, axes)))
+        approx(d, np.transpose(x, axes), 1e-2, 1e-1)
+    # should_quantize_symmetric_int8_permuted_batch_dims
+    x = grid(2048, (2, 4, 8, 32))
+    approx(np.transpose(roundtrip(np.ascontiguousarray(np.transpose(x, (1, 2, 0, 3))), per_tensor), (2, 0, 1, 3)), x, 1e-2, 1e-1)
+
+
 # ------------------------------------------------------------------ seeded parity, all schemes
 
 @pytest.mark.parametrize("value", [QuantValue.Q8S, QuantValue.Q4S])
@@ -517,12 +582,14 @@ def test_q_permute_matches_oracle(dev, value, store, block, shape, axes):
         pytest.skip("the source itself cannot be packed")
     tq = QTensorOps.quantize_dynamic(FloatOps.float_from_data(x, dev), scheme)
     q, s = unpack_blob(QTensorOps.q_into_data(tq))
-    if store == QuantStore.PackedU32 and new_last % nq:
-        with pytest.raises(ba.BurnqError):   # "Can't store in u32"
+    if store == QuantStore.PackedU32 and new_last % nq and value != QuantValue.Q8S:
+        with pytest.raises(ba.BurnqError):   # "Can't store in u32" (sub-byte values have no native store)
             QTensorOps.q_permute(tq, axes)
         return
     tp = QTensorOps.q_permute(tq, axes)
     assert tp.shape == tuple(shape[a] for a in axes)
+    # (a Q8S result whose last dim does not fill whole words comes back natively stored: same bytes)
+    assert tp.scheme.store == (QuantStore.Native if new_last % nq else store)
     qp, sp, bp = no.q_permute(q, s, list(block) if block else None, axes)
     blob = QTensorOps.q_into_data(tp)
     got_q, got_s = unpack_blob(blob)

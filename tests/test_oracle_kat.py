@@ -499,3 +499,37 @@ def test_two_level_properties_the_reference_asserts():
         return np.abs(t - co.dequantize(q, sch, eff)).sum() / np.abs(t).sum()
 
     assert abs(error(small) - error(big)) / error(big) < 0.2
+
+
+def test_scale_dtype_accuracy_as_the_reference_measures_it():
+    """crates/burn-backend-tests/tests/tensor/float/quantization/accuracy.rs:108-139 with its sample
+    generator (a 64-bit LCG through Box-Muller): Q8S, blocks of 32, [64, 64] of N(0, 1) -- f16 scales
+    are indistinguishable from f32 ones (relative error within 20 %); and, for the two-level scheme
+    (:88-106's remedy), the error at std 0.02 is that of f32 scales too."""
+    def normal_samples(n, std):
+        state, out = 0x2545F4914F6CDD1D, []
+        def uniform():
+            nonlocal state
+            state = (state * 6364136223846793005 + 1442695040888963407) & 0xFFFFFFFFFFFFFFFF
+            return (np.float32(state >> 40) + np.float32(0.5)) / np.float32(1 << 24)
+        for _ in range(n):
+            u1, u2 = uniform(), uniform()
+            r = np.sqrt(np.float32(-2.0) * np.log(u1))
+            out.append(r * np.cos(np.float32(2 * np.pi) * u2) * np.float32(std))
+        return np.float32(out).reshape(64, 64)
+
+    def rel_err(x, d):
+        return np.sqrt(((x.astype(np.float64) - d) ** 2).sum()) / np.sqrt((x.astype(np.float64) ** 2).sum())
+
+    sch = co.Scheme.make(co.Q8S, [32], co.STORE_NATIVE)
+    x = normal_samples(64 * 64, 1.0)
+    q, s = co.quantize_dynamic(x, sch)
+    f32_err = rel_err(x, co.dequantize(q, sch, s))
+    s16 = co.scale_to_dtype(s, co.SCALE_F16)
+    f16_err = rel_err(x, co.dequantize(co.quantize(x, sch, s16), sch, s16))
+    assert abs(f16_err - f32_err) / f32_err < 0.20
+    small = normal_samples(64 * 64, 0.02)
+    q, s = co.quantize_dynamic(small, sch)
+    exact = rel_err(small, co.dequantize(q, sch, s))
+    q2, _, _, eff = co.quantize_dynamic_two_level(small, sch, co.SCALE_F16)
+    assert abs(rel_err(small, co.dequantize(q2, sch, eff)) - exact) / exact < 0.20
