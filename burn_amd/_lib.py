@@ -23,7 +23,7 @@ F32, BF16, QFLOAT = 0, 1, 2
 Q8S, Q4S, Q2S = 0, 1, 2
 LEVEL_TENSOR, LEVEL_BLOCK = 0, 1
 STORE_NATIVE, STORE_PACKED_U32 = 0, 1
-SCALE_F32, SCALE_F16, SCALE_BF16 = 0, 1, 2
+SCALE_F32, SCALE_F16, SCALE_BF16, SCALE_UE4M3 = 0, 1, 2, 3
 
 
 class CScheme(C.Structure):

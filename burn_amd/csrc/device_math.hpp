@@ -28,13 +28,19 @@ __device__ __forceinline__ float scale_from_absmax(float amax, float span) {
 }
 
 // scale_to_dtype (crates/burn-std/src/tensor/quantization.rs:354-368): the smallest value the scale
-// dtype represents that is no smaller than s, as an f32. sdt: 0 f32 (identity), 1 f16, 2 bf16
-// (BQ_SCALE_*). NaN and the infinities pass through; a finite scale past the dtype's largest finite
-// value saturates to it.
+// dtype represents that is no smaller than s, as an f32. sdt: 0 f32 (identity), 1 f16, 2 bf16,
+// 3 ue4m3 (BQ_SCALE_*). NaN and the infinities pass through; a finite scale past the dtype's largest
+// finite value saturates to it.
 __device__ __forceinline__ float scale_round_up(float s, int sdt) {
   if (sdt == 0) return s;
   const uint32_t u = __float_as_uint(s), mag = u & 0x7FFFFFFFu;
   if (mag >= 0x7F800000u) return s;
+  if (sdt == 3) {  // ue4m3: 4 significant bits down to 2^-6, multiples of 2^-9 below; largest value 448; unsigned
+    if (!(s > 0.0f)) return 0.0f;
+    if (s < 0.015625f) return ceilf(s * 512.0f) * 0.001953125f;
+    const uint32_t r = (u & 0xFFFFFu) ? ((u | 0xFFFFFu) + 1u) : u;   // magnitude up to a multiple of 2^(e - 3)
+    return r > 0x43E00000u ? 448.0f : __uint_as_float(r);
+  }
   if (sdt == 2) {  // bf16: the upper 16 bits; rounding the magnitude up (s > 0) or truncating it (s < 0)
     if ((u & 0xFFFFu) == 0u) return s;
     if (u & 0x80000000u) return __uint_as_float(u & 0xFFFF0000u);

@@ -172,7 +172,8 @@ void write_scheme(CborWriter& w, const bq_scheme& s) {
   else { w.map(1); w.text("Block"); w.array(s.block_rank); for (int i = 0; i < s.block_rank; ++i) w.uint(s.block[i]); }
   w.text("store");
   if (s.store == BQ_STORE_NATIVE) { w.text("Native"); } else { w.map(1); w.text("PackedU32"); w.uint(0); }
-  w.text("scale_dtype"); w.text(s.scale_dtype == BQ_SCALE_F32 ? "F32" : s.scale_dtype == BQ_SCALE_F16 ? "F16" : "BF16");
+  w.text("scale_dtype");
+  w.text(s.scale_dtype == BQ_SCALE_F32 ? "F32" : s.scale_dtype == BQ_SCALE_F16 ? "F16" : s.scale_dtype == BQ_SCALE_BF16 ? "BF16" : "UE4M3");
   w.text("mode"); w.text("Symmetric");
   if (s.tensor_scale) { w.text("tensor_scale"); w.text("F32"); }  // two-level: a per-tensor f32 scale on top
 }
@@ -189,7 +190,8 @@ bool read_scheme(const Cbor& c, bq_scheme* s) {
     s->tensor_scale = 1;
   }
   if (sd->s == "F32") s->scale_dtype = BQ_SCALE_F32; else if (sd->s == "F16") s->scale_dtype = BQ_SCALE_F16;
-  else if (sd->s == "BF16") s->scale_dtype = BQ_SCALE_BF16; else return false;
+  else if (sd->s == "BF16") s->scale_dtype = BQ_SCALE_BF16; else if (sd->s == "UE4M3") s->scale_dtype = BQ_SCALE_UE4M3;
+  else return false;
   if (level->kind == Cbor::Text && level->s == "Tensor") {
     s->level = BQ_LEVEL_TENSOR;
   } else if (level->kind == Cbor::Map && level->get("Block") && level->get("Block")->kind == Cbor::Array) {

@@ -547,18 +547,42 @@ __device__ __forceinline__ float f16_bits_to_f32(uint16_t h) {
   return __uint_as_float(sign | ((ex + 112u) << 23) | (man << 13));
 }
 
-__global__ void scales_to_wire_kernel(const float* __restrict__ src, uint16_t* __restrict__ dst, size_t n, int sdt) {
+// e4m3 bits of a value the format represents exactly (non-negative half; NaN and infinities -> 0x7F)
+__device__ __forceinline__ uint8_t e4m3_bits_exact(float v) {
+  const uint32_t u = __float_as_uint(v);
+  if ((u & 0x7FFFFFFFu) >= 0x7F800000u) return 0x7Fu;
+  if (!(v > 0.0f)) return 0u;
+  if (v < 0.015625f) return static_cast<uint8_t>(v * 512.0f);          // subnormal: m = v / 2^-9
+  return static_cast<uint8_t>((((u >> 23) - 127u + 7u) << 3) | ((u >> 20) & 7u));
+}
+__device__ __forceinline__ float e4m3_bits_to_f32(uint8_t b) {
+  const uint32_t ex = (b >> 3) & 0xFu, man = b & 7u;
+  if (ex == 15u && man == 7u) return __uint_as_float(0x7FC00000u);
+  const float v = ex == 0u ? static_cast<float>(man) * 0.001953125f : __uint_as_float(((ex + 120u) << 23) | (man << 20));
+  return (b & 0x80u) ? -v : v;
+}
+
+// T: uint16_t (f16, bf16) or uint8_t (ue4m3)
+template <typename T>
+__global__ void scales_to_wire_kernel(const float* __restrict__ src, T* __restrict__ dst, size_t n, int sdt) {
   const size_t i = static_cast<size_t>(blockIdx.x) * blockDim.x + threadIdx.x;
   if (i >= n) return;
   // (a scale that did not pass through scale_round_up, e.g. given by hand: rounded up here as well)
   const float v = scale_round_up(src[i], sdt);
-  dst[i] = sdt == 2 ? static_cast<uint16_t>(__float_as_uint(v) >> 16) : f16_bits_exact(v);
+  if (sizeof(T) == 1)
+    dst[i] = static_cast<T>(e4m3_bits_exact(v));
+  else
+    dst[i] = static_cast<T>(sdt == 2 ? static_cast<uint16_t>(__float_as_uint(v) >> 16) : f16_bits_exact(v));
 }
 
-__global__ void scales_from_wire_kernel(const uint16_t* __restrict__ src, float* __restrict__ dst, size_t n, int sdt) {
+template <typename T>
+__global__ void scales_from_wire_kernel(const T* __restrict__ src, float* __restrict__ dst, size_t n, int sdt) {
   const size_t i = static_cast<size_t>(blockIdx.x) * blockDim.x + threadIdx.x;
   if (i >= n) return;
-  dst[i] = sdt == 2 ? __uint_as_float(static_cast<uint32_t>(src[i]) << 16) : f16_bits_to_f32(src[i]);
+  if (sizeof(T) == 1)
+    dst[i] = e4m3_bits_to_f32(static_cast<uint8_t>(src[i]));
+  else
+    dst[i] = sdt == 2 ? __uint_as_float(static_cast<uint32_t>(src[i]) << 16) : f16_bits_to_f32(static_cast<uint16_t>(src[i]));
 }
 
 bq_status launch_scale_from_cells(const uint32_t* cells, int value, int sdt, float* scale_out, hipStream_t st) {
@@ -600,12 +624,12 @@ __global__ void scales_times_global_kernel(const float* __restrict__ stored, con
 
 bq_status launch_two_level_split(float* scales, size_t n, const uint32_t* cells, int sdt, float* global_out, float* stored,
                                  hipStream_t st) {
-  if (sdt != BQ_SCALE_F16)
+  if (sdt != BQ_SCALE_F16 && sdt != BQ_SCALE_UE4M3)
     BQ_FAIL(BQ_ERR_UNSUPPORTED_SCHEME,
-            "block scales of this dtype reach f32's range, which a per-tensor scale cannot absorb (f16 block scales can)");
+            "block scales of this dtype reach f32's range, which a per-tensor scale cannot absorb (f16 and ue4m3 block scales can)");
   if (n == 0) return BQ_OK;
   hipLaunchKernelGGL(two_level_split_kernel, dim3(static_cast<unsigned>((n + kThreads - 1) / kThreads)), dim3(kThreads), 0, st,
-                     scales, n, cells, 65504.0f, sdt, global_out, stored);
+                     scales, n, cells, sdt == BQ_SCALE_F16 ? 65504.0f : 448.0f, sdt, global_out, stored);
   BQ_HIP(hipGetLastError());
   return BQ_OK;
 }
@@ -627,16 +651,22 @@ bq_status launch_round_scales(const float* src, float* dst, size_t n, int sdt, h
 
 bq_status launch_scales_to_wire(const float* src, void* dst, size_t n, int sdt, hipStream_t st) {
   if (n == 0) return BQ_OK;
-  hipLaunchKernelGGL(scales_to_wire_kernel, dim3(static_cast<unsigned>((n + 255) / 256)), dim3(256), 0, st, src,
-                     static_cast<uint16_t*>(dst), n, sdt);
+  const dim3 grid(static_cast<unsigned>((n + 255) / 256));
+  if (sdt == BQ_SCALE_UE4M3)
+    hipLaunchKernelGGL(scales_to_wire_kernel<uint8_t>, grid, dim3(256), 0, st, src, static_cast<uint8_t*>(dst), n, sdt);
+  else
+    hipLaunchKernelGGL(scales_to_wire_kernel<uint16_t>, grid, dim3(256), 0, st, src, static_cast<uint16_t*>(dst), n, sdt);
   BQ_HIP(hipGetLastError());
   return BQ_OK;
 }
 
 bq_status launch_scales_from_wire(const void* src, float* dst, size_t n, int sdt, hipStream_t st) {
   if (n == 0) return BQ_OK;
-  hipLaunchKernelGGL(scales_from_wire_kernel, dim3(static_cast<unsigned>((n + 255) / 256)), dim3(256), 0, st,
-                     static_cast<const uint16_t*>(src), dst, n, sdt);
+  const dim3 grid(static_cast<unsigned>((n + 255) / 256));
+  if (sdt == BQ_SCALE_UE4M3)
+    hipLaunchKernelGGL(scales_from_wire_kernel<uint8_t>, grid, dim3(256), 0, st, static_cast<const uint8_t*>(src), dst, n, sdt);
+  else
+    hipLaunchKernelGGL(scales_from_wire_kernel<uint16_t>, grid, dim3(256), 0, st, static_cast<const uint16_t*>(src), dst, n, sdt);
   BQ_HIP(hipGetLastError());
   return BQ_OK;
 }

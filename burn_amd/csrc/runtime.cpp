@@ -59,7 +59,9 @@ static size_t value_bytes(const bq_scheme& s, const size_t* shape, int rank) {
 }
 
 // scale_size (crates/burn-std/src/tensor/quantization.rs:409-416): bytes per stored scale on the wire.
-static size_t scale_size(const bq_scheme& s) { return s.scale_dtype == BQ_SCALE_F32 ? 4 : 2; }
+static size_t scale_size(const bq_scheme& s) {
+  return s.scale_dtype == BQ_SCALE_F32 ? 4 : (s.scale_dtype == BQ_SCALE_UE4M3 ? 1 : 2);
+}
 // global_scale_size (same file): the f32 per-tensor scale a two-level scheme stores behind its block scales.
 static size_t global_size(const bq_scheme& s) { return s.tensor_scale ? 4 : 0; }
 
@@ -70,8 +72,8 @@ static bq_status check_scheme(const bq_scheme& s, const size_t* shape, int rank,
   if (rank < 1 || rank > BQ_MAX_RANK) BQ_FAIL(BQ_ERR_SHAPE, "rank %d outside 1..%d", rank, BQ_MAX_RANK);
   if (!value_supported(s.value))
     BQ_FAIL(BQ_ERR_UNSUPPORTED_SCHEME, "Quantization not supported for value %d (Q8S, Q4S and Q2S are)", s.value);
-  if (s.scale_dtype != BQ_SCALE_F32 && s.scale_dtype != BQ_SCALE_F16 && s.scale_dtype != BQ_SCALE_BF16)
-    BQ_FAIL(BQ_ERR_UNSUPPORTED_SCHEME, "scale dtype %d is not supported (f32, f16 and bf16 are)", s.scale_dtype);
+  if (s.scale_dtype > BQ_SCALE_UE4M3)
+    BQ_FAIL(BQ_ERR_UNSUPPORTED_SCHEME, "scale dtype %d is not supported (f32, f16, bf16 and ue4m3 are)", s.scale_dtype);
   if (s.level != BQ_LEVEL_TENSOR && s.level != BQ_LEVEL_BLOCK)
     BQ_FAIL(BQ_ERR_UNSUPPORTED_SCHEME, "unknown quantization level %d", s.level);
   if (s.tensor_scale > 1 || (s.tensor_scale && s.level != BQ_LEVEL_BLOCK))
@@ -625,12 +627,12 @@ extern "C" bq_status bq_q_from_data(bq_device* dev, const uint8_t* bytes, size_t
   if (e == hipSuccess && ssz == 4) {
     e = hipMemcpyAsync(scales_dst, bytes + t->value_bytes, 4 * t->num_scales, hipMemcpyHostToDevice, dev->stream);
   } else if (e == hipSuccess) {
-    // 2-byte scales: staged in a device block, widened (exactly) to the f32 the kernels read
+    // 2- and 1-byte scales: staged in a device block, widened (exactly) to the f32 the kernels read
     void* stage = nullptr;
     size_t stage_bytes = 0;
-    rc = dev->alloc(2 * t->num_scales, &stage, &stage_bytes);
+    rc = dev->alloc(ssz * t->num_scales, &stage, &stage_bytes);
     if (rc == BQ_OK) {
-      e = hipMemcpyAsync(stage, bytes + t->value_bytes, 2 * t->num_scales, hipMemcpyHostToDevice, dev->stream);
+      e = hipMemcpyAsync(stage, bytes + t->value_bytes, ssz * t->num_scales, hipMemcpyHostToDevice, dev->stream);
       if (e == hipSuccess) rc = launch_scales_from_wire(stage, scales_dst, t->num_scales, scheme->scale_dtype, dev->stream);
       dev->release(stage, stage_bytes);  // (stream ordered: the next owner's work queues behind the kernel)
     }
@@ -676,10 +678,10 @@ extern "C" bq_status bq_q_into_data(const bq_tensor* t, uint8_t* bytes, size_t c
   }
   void* stage = nullptr;
   size_t stage_bytes = 0;
-  BQ_TRY(t->dev->alloc(2 * t->num_scales, &stage, &stage_bytes));
+  BQ_TRY(t->dev->alloc(ssz * t->num_scales, &stage, &stage_bytes));
   bq_status rc = launch_scales_to_wire(scales_src, stage, t->num_scales, t->scheme.scale_dtype, st);
   hipError_t e = hipSuccess;
-  if (rc == BQ_OK) e = hipMemcpyAsync(bytes + t->value_bytes, stage, 2 * t->num_scales, hipMemcpyDeviceToHost, st);
+  if (rc == BQ_OK) e = hipMemcpyAsync(bytes + t->value_bytes, stage, ssz * t->num_scales, hipMemcpyDeviceToHost, st);
   if (e == hipSuccess) e = hipStreamSynchronize(st);
   t->dev->release(stage, stage_bytes);
   if (e != hipSuccess) BQ_FAIL(BQ_ERR_HIP, "device to host copy failed: %s", hipGetErrorString(e));
@@ -739,9 +741,9 @@ static bq_status quantize_impl(const bq_tensor* x, const bq_scheme* scheme, cons
   if (global != nullptr && (global->dtype != BQ_F32 || global->numel() != 1 || global->dev != x->dev))
     BQ_FAIL(BQ_ERR_SHAPE, "the per-tensor scale must be an f32 tensor of one element on the input's device");
   // (normalize_scales, crates/burn-backend/src/quantization/scheme.rs:115-118)
-  if (dynamic && two_level && scheme->scale_dtype != BQ_SCALE_F16)
+  if (dynamic && two_level && scheme->scale_dtype != BQ_SCALE_F16 && scheme->scale_dtype != BQ_SCALE_UE4M3)
     BQ_FAIL(BQ_ERR_UNSUPPORTED_SCHEME,
-            "block scales of this dtype reach f32's range, which a per-tensor scale cannot absorb (f16 block scales can)");
+            "block scales of this dtype reach f32's range, which a per-tensor scale cannot absorb (f16 and ue4m3 block scales can)");
   bq_tensor* q = nullptr;
   BQ_TRY(new_quantized(x->dev, *scheme, x->shape, x->rank, &q));
   if (!dynamic) {

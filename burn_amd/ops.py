@@ -215,6 +215,17 @@ class FloatOps:
         return _wrap(h, lhs.device)
 
 
+def f32_from_e4m3_bits(bits) -> np.ndarray:
+    """OCP e4m3 bytes -> f32, exactly (e4m3::from_bits(b).to_f32(),
+    crates/burn-std/src/tensor/quantization.rs:437): bias 7, 3 mantissa bits, subnormals m * 2^-9,
+    0x7F / 0xFF NaN."""
+    b = np.asarray(bits, np.uint8).astype(np.int64)
+    e, m = (b >> 3) & 0xF, b & 7
+    v = np.where(e == 0, m * 2.0 ** -9, (1 + m / 8.0) * 2.0 ** (e.astype(np.float64) - 7))
+    v = np.where((e == 15) & (m == 7), np.nan, v)
+    return np.where(b & 0x80, -v, v).astype(np.float32)
+
+
 class TensorData:
     """bytes + shape + scheme: the QFloat TensorData blob (values || block scales, dense)."""
 
@@ -251,6 +262,8 @@ class TensorData:
             scales = raw.copy().view(np.float32)
         elif self.scheme.scale_dtype == ScaleDtype.F16:
             scales = raw.copy().view(np.float16).astype(np.float32)
+        elif self.scheme.scale_dtype == ScaleDtype.UE4M3:
+            scales = f32_from_e4m3_bits(raw)
         else:
             scales = f32_from_bf16_bits(raw.copy().view(np.uint16))
         return self.bytes[:cut], scales.reshape(pshape)

@@ -2,7 +2,7 @@
 
 `QuantScheme` mirrors cubecl_common::quant::scheme::QuantScheme as burn re-exports it
 (crates/burn-std/src/tensor/quantization.rs:4-6), restricted to what this backend implements:
-symmetric Q8S / Q4S / Q2S values, per-tensor or per-block scales stored as f32, f16 or bf16, an
+symmetric Q8S / Q4S / Q2S values, per-tensor or per-block scales stored as f32, f16, bf16 or ue4m3, an
 optional f32 per-tensor scale on top of block scales (two-level), Native or PackedU32(0) store.
 """
 from __future__ import annotations
@@ -35,10 +35,11 @@ class ScaleDtype(IntEnum):
     F32 = _lib.SCALE_F32
     F16 = _lib.SCALE_F16
     BF16 = _lib.SCALE_BF16
+    UE4M3 = _lib.SCALE_UE4M3   # one byte: the non-negative half of OCP e4m3
 
     def size(self) -> int:
         """scale_size -- crates/burn-std/src/tensor/quantization.rs:409-416."""
-        return 4 if self == ScaleDtype.F32 else 2
+        return {ScaleDtype.F32: 4, ScaleDtype.UE4M3: 1}.get(self, 2)
 
 
 @dataclass(frozen=True)

@@ -61,10 +61,10 @@ enum { BQ_F32 = 0, BQ_BF16 = 1, BQ_QFLOAT = 2 };
 enum { BQ_Q8S = 0, BQ_Q4S = 1, BQ_Q2S = 2 };
 enum { BQ_LEVEL_TENSOR = 0, BQ_LEVEL_BLOCK = 1 };
 enum { BQ_STORE_NATIVE = 0, BQ_STORE_PACKED_U32 = 1 };
-/* ScaleDtype. F16 / BF16: the quantizer divides by the scale rounded UP to the scale dtype
+/* ScaleDtype. F16 / BF16 / UE4M3: the quantizer divides by the scale rounded UP to the scale dtype
  * (scale_to_dtype, crates/burn-std/src/tensor/quantization.rs:354-368) and the blob stores 2 bytes
- * per scale (encode_scales, same file). */
-enum { BQ_SCALE_F32 = 0, BQ_SCALE_F16 = 1, BQ_SCALE_BF16 = 2 };
+ * (UE4M3: 1 byte, the non-negative half of OCP e4m3) per scale (encode_scales, same file). */
+enum { BQ_SCALE_F32 = 0, BQ_SCALE_F16 = 1, BQ_SCALE_BF16 = 2, BQ_SCALE_UE4M3 = 3 };
 
 /* The fields of QuantScheme this path reads. `block` holds block_rank extents aligned to the
  * trailing dims (BlockSize::to_dim_vec pads the leading dims with 1). PackedU32 always packs
@@ -73,7 +73,7 @@ typedef struct bq_scheme {
   uint8_t value;       /* BQ_Q8S | BQ_Q4S | BQ_Q2S */
   uint8_t level;       /* BQ_LEVEL_TENSOR | BQ_LEVEL_BLOCK */
   uint8_t store;       /* BQ_STORE_NATIVE (Q8S only) | BQ_STORE_PACKED_U32 */
-  uint8_t scale_dtype; /* BQ_SCALE_F32 | BQ_SCALE_F16 | BQ_SCALE_BF16 */
+  uint8_t scale_dtype; /* BQ_SCALE_F32 | BQ_SCALE_F16 | BQ_SCALE_BF16 | BQ_SCALE_UE4M3 */
   uint8_t block_rank;
   uint8_t tensor_scale; /* block level only: 1 = an f32 per-tensor scale on top of the block scales (below) */
   uint8_t reserved[2];
@@ -85,7 +85,7 @@ typedef struct bq_scheme {
  * (QuantizedBytes::new, same file :245-266). quantize_dynamic splits the block scales so that the
  * largest lands on the scale dtype's largest value (normalize_scales,
  * crates/burn-backend/src/quantization/scheme.rs:106-134), which the reference allows for scale
- * dtypes whose largest value does not exceed f16's: here that is BQ_SCALE_F16. */
+ * dtypes whose largest value does not exceed f16's: BQ_SCALE_F16 and BQ_SCALE_UE4M3. */
 
 typedef struct bq_device bq_device; /* one GPU: stream, allocation cache, workspace */
 typedef struct bq_tensor bq_tensor; /* ref-counted device tensor: float, or values || scales */

@@ -492,8 +492,44 @@ static uint16_t bf16_from_f32_rne(float f) {
   return (uint16_t)(u >> 16);
 }
 
+/* e4m3 (OCP FP8 E4M3: 4 exponent bits, bias 7, 3 mantissa bits, no infinities, 0x7F = NaN, largest
+ * value 0x7E = 448; subnormals m * 2^-9). "UE4M3" uses the non-negative half. */
+static float f32_from_e4m3(uint8_t b) {
+  const uint32_t ex = (b >> 3) & 0xFu, man = b & 7u;
+  float v;
+  if (ex == 0) v = (float)man * 0.001953125f;                       /* m * 2^-9 */
+  else if (ex == 15 && man == 7) return NAN;
+  else v = ldexpf(1.0f + (float)man * 0.125f, (int)ex - 7);
+  return (b & 0x80u) ? -v : v;
+}
+/* bits of a value that e4m3 represents exactly (what the rounding below returns) */
+static uint8_t e4m3_bits_exact(float v) {
+  if (v != v) return 0x7Fu;
+  if (v <= 0.0f) return 0;
+  if (v < 0.015625f) return (uint8_t)(v * 512.0f);                  /* subnormal: m = v / 2^-9 */
+  int e;
+  const float m = frexpf(v, &e);                                    /* v = m * 2^e, m in [0.5, 1) */
+  if (v > 448.0f) return 0x7Eu;
+  return (uint8_t)(((unsigned)(e - 1 + 7) << 3) | (unsigned)((m * 2.0f - 1.0f) * 8.0f));
+}
+/* smallest non-negative e4m3 value that is no smaller than s (s > 0, finite) */
+static float e4m3_round_up(float s) {
+  if (s < 0.015625f) {                                              /* below the smallest normal, 2^-6 */
+    return ceilf(s * 512.0f) * 0.001953125f;
+  }
+  int e;
+  (void)frexpf(s, &e);                                              /* s in [2^(e-1), 2^e) */
+  const float step = ldexpf(1.0f, e - 1 - 3);                       /* spacing of e4m3 values there */
+  float r = ceilf(s / step) * step;                                 /* exact: s / step < 16 */
+  return r > 448.0f ? 448.0f : r;                                   /* saturates (parity unpinned) */
+}
+
 float bqo_scale_to_dtype(float scale, int dtype) {
   if (dtype == BQO_SCALE_F32) return scale;
+  if (dtype == BQO_SCALE_UE4M3) {
+    if (scale != scale || scale == INFINITY) return scale;
+    return scale > 0.0f ? e4m3_round_up(scale) : 0.0f;              /* unsigned: nothing below zero */
+  }
   if (scale != scale || scale == INFINITY || scale == -INFINITY) return scale;
   /* start from the nearest representable value, step up while it is below the scale */
   if (dtype == BQO_SCALE_F16) {
@@ -518,7 +554,7 @@ float bqo_scale_to_dtype(float scale, int dtype) {
   return back;
 }
 
-size_t bqo_scale_size(int dtype) { return dtype == BQO_SCALE_F32 ? 4 : 2; }
+size_t bqo_scale_size(int dtype) { return dtype == BQO_SCALE_F32 ? 4 : (dtype == BQO_SCALE_UE4M3 ? 1 : 2); }
 
 /* normalize_scales (burn-backend/src/quantization/scheme.rs:106-134): the per-tensor scale of a
  * two-level scheme is the largest block scale over the block dtype's largest value, kept at or
@@ -527,10 +563,11 @@ size_t bqo_scale_size(int dtype) { return dtype == BQO_SCALE_F32 ? 4 : 2; }
  * per-tensor scale, or NaN for a block dtype the reference refuses (its largest value must not
  * exceed f16's: of f32 / f16 / bf16 that leaves f16, largest value 65504). */
 float bqo_normalize_scales(float* scales, size_t n, int block_dtype) {
-  if (block_dtype != BQO_SCALE_F16) return NAN;
+  if (block_dtype != BQO_SCALE_F16 && block_dtype != BQO_SCALE_UE4M3) return NAN;
+  const float dtype_max = block_dtype == BQO_SCALE_F16 ? 65504.0f : 448.0f;
   float top = scales[0];
   for (size_t i = 1; i < n; ++i) top = scales[i] > top ? scales[i] : top;
-  float global = top / 65504.0f;
+  float global = top / dtype_max;
   if (global < 1.17549435e-38f) global = 1.17549435e-38f;   /* f32::MIN_POSITIVE */
   for (size_t i = 0; i < n; ++i) scales[i] = scales[i] / global;
   return global;
@@ -551,6 +588,10 @@ void bqo_encode_scales(const float* scales, size_t n, int dtype, uint8_t* out) {
   for (size_t i = 0; i < n; ++i) {
     if (dtype == BQO_SCALE_F32) {
       memcpy(out + 4 * i, scales + i, 4);
+    } else if (dtype == BQO_SCALE_UE4M3) {
+      /* (scales reach the codec already rounded up to the dtype, burn-ndarray/src/ops/qtensor.rs:90-95:
+       * whatever rounding e4m3::from_f32 applies, it returns such a value unchanged) */
+      out[i] = e4m3_bits_exact(bqo_scale_to_dtype(scales[i], dtype));
     } else {
       uint16_t h = dtype == BQO_SCALE_F16 ? f16_from_f32_rne(scales[i]) : bf16_from_f32_rne(scales[i]);
       memcpy(out + 2 * i, &h, 2);
@@ -562,6 +603,8 @@ void bqo_decode_scales(const uint8_t* in, size_t n, int dtype, float* out) {
   for (size_t i = 0; i < n; ++i) {
     if (dtype == BQO_SCALE_F32) {
       memcpy(out + i, in + 4 * i, 4);
+    } else if (dtype == BQO_SCALE_UE4M3) {
+      out[i] = f32_from_e4m3(in[i]);
     } else {
       uint16_t h;
       memcpy(&h, in + 2 * i, 2);

@@ -37,9 +37,19 @@
  *                        the f32 neighbour above goes to the next representable value, the one
  *                        below stays) and by the reference test's own scales and properties
  *                        (:631-657: rounded >= scale, the codec leaves a rounded scale alone).
+ *                        UE4M3 (one byte, the non-negative half of OCP e4m3: bias 7, 3 mantissa
+ *                        bits, subnormals m * 2^-9, largest value 448, 0x7F NaN; decoded as the
+ *                        reference does, e4m3::from_bits().to_f32(), :437): the same rule over its
+ *                        127 values, brute force over all of them, and the inequalities the
+ *                        reference's accuracy and two-level tests assert (accuracy.rs:88-139,
+ *                        ops/quantize.rs:238-290, scheme.rs:50-123), which fail if scales are
+ *                        rounded down, flushed below 2^-6 or left unsaturated.
  *                        PARITY UNPINNED: what a finite scale beyond the dtype's largest finite
  *                        value becomes (this restatement saturates to it, as the reference's test
- *                        comment says of e4m3), and UE4M3 / UE8M0 (not implemented).
+ *                        comment says of e4m3), what the codec writes for a value the dtype does
+ *                        not represent (never produced by quantize: scales are rounded up first;
+ *                        here such a value is rounded up as well), and UE8M0 (unimplemented in the
+ *                        reference itself, :439).
  *   bqo_encode/decode_scales  same test (:631-657) and the two-level layout test (:659-684).
  *   bqo_normalize_scales, bqo_two_level_scales  restated step for step from the reference's tensor
  *                        ops; no reference-held numbers exist. Pinned by what the mathematics
@@ -73,7 +83,7 @@ extern "C" {
 enum { BQO_Q8S = 0, BQO_Q4S = 1, BQO_Q2S = 2 }; /* QuantValue (symmetric signed ints only); Q2S = ternary */
 enum { BQO_LEVEL_TENSOR = 0, BQO_LEVEL_BLOCK = 1 };
 enum { BQO_STORE_NATIVE = 0, BQO_STORE_PACKED_U32 = 1 };
-enum { BQO_SCALE_F32 = 0, BQO_SCALE_F16 = 1, BQO_SCALE_BF16 = 2 };   /* ScaleDtype */
+enum { BQO_SCALE_F32 = 0, BQO_SCALE_F16 = 1, BQO_SCALE_BF16 = 2, BQO_SCALE_UE4M3 = 3 };   /* ScaleDtype */
 
 /* Mirrors the fields of cubecl_common::quant::scheme::QuantScheme that this path reads. */
 typedef struct {

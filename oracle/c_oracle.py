@@ -275,7 +275,7 @@ def max_threads():
     return lib().bqo_max_threads()
 
 
-SCALE_F32, SCALE_F16, SCALE_BF16 = 0, 1, 2
+SCALE_F32, SCALE_F16, SCALE_BF16, SCALE_UE4M3 = 0, 1, 2, 3
 
 
 def scale_to_dtype(scales, dtype):

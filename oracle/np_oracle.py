@@ -182,7 +182,23 @@ def scale_to_dtype(scales, dtype="F32"):
         r = np.where(np.isfinite(s) & ((r & 0x7FFFFFFF) >= 0x7F800000), (r & 0x80000000) | 0x7F7F0000, r)
         r = np.where(np.isfinite(s), r, u)
         return r.astype(np.uint32).view(np.float32)
+    if dtype == "UE4M3":
+        # the 127 non-negative e4m3 values in ascending order, then a search: an independent route
+        # to "the smallest representable value that is no smaller"
+        table = ue4m3_values()
+        idx = np.searchsorted(table, s.astype(np.float64), side="left")
+        out = table[np.minimum(idx, table.size - 1)].astype(np.float32)      # past 448: saturates
+        out = np.where(s > 0, out, np.float32(0))
+        return np.where(np.isfinite(s), out, s).astype(np.float32)
     raise ValueError(dtype)
+
+
+def ue4m3_values():
+    """Every value of the non-negative half of OCP e4m3 (bits 0x00 .. 0x7E), ascending, as float64:
+    m * 2^-9 for exponent field 0, (1 + m/8) * 2^(e - 7) otherwise."""
+    bits = np.arange(0x7F)
+    e, m = bits >> 3, bits & 7
+    return np.where(e == 0, m * 2.0 ** -9, (1 + m / 8.0) * 2.0 ** (e.astype(np.float64) - 7))
 
 
 def quantize_dynamic_two_level(x, value="Q8S", block=None, block_dtype="F16"):
@@ -191,11 +207,12 @@ def quantize_dynamic_two_level(x, value="Q8S", block=None, block_dtype="F16"):
     NdArray::quantize against global * scale_to_dtype(relative block scale)
     (crates/burn-ndarray/src/ops/qtensor.rs:90-101, 519-531).
     -> (values, stored block scales, global, effective scales)."""
-    if block_dtype != "F16":
+    if block_dtype not in ("F16", "UE4M3"):
         raise ValueError("block scales of this dtype reach f32's range, which a per-tensor scale cannot absorb")
+    top = np.float32(65504.0 if block_dtype == "F16" else 448.0)
     lo, hi = compute_range(x, block)
     scales = compute_q_params(lo, hi, value).astype(np.float32)
-    g = np.maximum(np.float32(scales.max()) / np.float32(65504.0), np.float32(1.17549435e-38)).astype(np.float32)
+    g = np.maximum(np.float32(scales.max()) / top, np.float32(1.17549435e-38)).astype(np.float32)
     rel = (scales / g).astype(np.float32)
     stored = scale_to_dtype(rel, block_dtype)
     eff = (g * stored).astype(np.float32)

@@ -736,7 +736,7 @@ def test_validate_mode_fails_where_the_reference_panics(dev):
 
 # ------------------------------------------------------------------ f16 / bf16 scales
 
-SDT = {ScaleDtype.F16: (co.SCALE_F16, "F16"), ScaleDtype.BF16: (co.SCALE_BF16, "BF16")}
+SDT = {ScaleDtype.F16: (co.SCALE_F16, "F16"), ScaleDtype.BF16: (co.SCALE_BF16, "BF16"), ScaleDtype.UE4M3: (co.SCALE_UE4M3, "UE4M3")}
 
 
 def check_scale_dtype(dev, x, scheme, given_scales=None):
@@ -769,7 +769,7 @@ def check_scale_dtype(dev, x, scheme, given_scales=None):
     return tq, q_ref, s_ref
 
 
-@pytest.mark.parametrize("sdt", [ScaleDtype.F16, ScaleDtype.BF16])
+@pytest.mark.parametrize("sdt", [ScaleDtype.F16, ScaleDtype.BF16, ScaleDtype.UE4M3])
 @pytest.mark.parametrize("value", [QuantValue.Q8S, QuantValue.Q4S])
 @pytest.mark.parametrize("block", [None, (32,), (16,), (2, 32)])
 def test_quantize_with_two_byte_scales(dev, sdt, value, block):
@@ -787,7 +787,7 @@ def test_quantize_with_two_byte_scales(dev, sdt, value, block):
     check_scale_dtype(dev, x, scheme, given_scales=given)
 
 
-@pytest.mark.parametrize("sdt", [ScaleDtype.F16, ScaleDtype.BF16])
+@pytest.mark.parametrize("sdt", [ScaleDtype.F16, ScaleDtype.BF16, ScaleDtype.UE4M3])
 def test_two_byte_scales_over_the_exponent_range(dev, sdt):
     """Blocks whose scale runs from far below the format's subnormals to past its largest value."""
     rng = np.random.default_rng(12)
@@ -797,7 +797,7 @@ def test_two_byte_scales_over_the_exponent_range(dev, sdt):
     check_scale_dtype(dev, x[20], QuantScheme(store=QuantStore.Native, scale_dtype=sdt))
 
 
-@pytest.mark.parametrize("sdt", [ScaleDtype.F16, ScaleDtype.BF16])
+@pytest.mark.parametrize("sdt", [ScaleDtype.F16, ScaleDtype.BF16, ScaleDtype.UE4M3])
 def test_q_matmul_with_two_byte_scales(dev, sdt):
     rng = np.random.default_rng(8)
     w = (rng.standard_normal((512, 384)) * 0.02).astype(np.float32)
@@ -825,22 +825,23 @@ def two_level_parts(blob: TensorData):
                                          (QuantValue.Q4S, QuantStore.PackedU32)])
 @pytest.mark.parametrize("shape,block,mag", [((16, 16), (2, 16), 1.0), ((64, 256), (32,), 0.02), ((4, 6, 32), (1, 2, 16), 300.0),
                                              ((128, 512), (64,), 1e-6), ((8, 64), (8,), 5.0)])
-def test_two_level_quantize_dynamic(dev, value, store, shape, block, mag):
+@pytest.mark.parametrize("sdt", [ScaleDtype.F16, ScaleDtype.UE4M3])
+def test_two_level_quantize_dynamic(dev, sdt, value, store, shape, block, mag):
     """f16 block scales under an f32 per-tensor scale (`.per_block(b, F16).per_tensor(F32)`): values,
     stored block scales, the per-tensor scale, the blob and the dequantized floats, all bit for bit
     against the oracle; and the blob read back gives the same tensor (the reference's round trip,
     crates/burn-backend-tests/tests/tensor/float/quantization/ops/quantize.rs:489-516)."""
     x = (np.random.default_rng(len(shape) * 100 + shape[-1]).standard_normal(shape) * mag).astype(np.float32)
-    scheme = QuantScheme(value=value, store=store).per_block(block, ScaleDtype.F16).per_tensor(ScaleDtype.F32)
+    scheme = QuantScheme(value=value, store=store).per_block(block, sdt).per_tensor(ScaleDtype.F32)
     assert scheme.tensor_scale == ScaleDtype.F32 and scheme.block == block
-    osch = oscheme(scheme)
-    q_ref, stored_ref, g_ref, eff_ref = co.quantize_dynamic_two_level(x, osch, co.SCALE_F16)
+    osch, code = oscheme(scheme), SDT[sdt][0]
+    q_ref, stored_ref, g_ref, eff_ref = co.quantize_dynamic_two_level(x, osch, code)
     tq = QTensorOps.quantize_dynamic(FloatOps.float_from_data(x, dev), scheme)
     assert tq.scheme == scheme
     blob = QTensorOps.q_into_data(tq)
     q, stored, g = two_level_parts(blob)
     assert g == g_ref and stored.tobytes() == stored_ref.tobytes() and (q == q_ref).all()
-    assert blob.bytes.tobytes() == co.encode_two_level(q_ref, osch, stored_ref, g_ref, co.SCALE_F16).tobytes()
+    assert blob.bytes.tobytes() == co.encode_two_level(q_ref, osch, stored_ref, g_ref, code).tobytes()
     assert blob.bytes.size == TensorData.data_len(shape, scheme)
     d_ref = co.dequantize(q_ref, osch, eff_ref)
     assert FloatOps.float_into_data(QTensorOps.dequantize(tq)).tobytes() == d_ref.tobytes()
@@ -864,6 +865,25 @@ def test_two_level_reference_cases(dev, approx):
     expected = x.astype(np.float64) @ direct.astype(np.float64)
     actual = FloatOps.float_into_data(QTensorOps.q_matmul(FloatOps.float_from_data(x, dev), tq))
     approx(actual, expected, 1e-2, 0)
+    # quantize.rs:213-236 and 238-290 as they stand, with ue4m3 block scales: exact round trip through
+    # the blob; the error is the same at either magnitude; one-level 8-bit scales degrade on small weights
+    ue = QuantScheme(store=QuantStore.Native).per_block((2, 16), ScaleDtype.UE4M3)
+    two, one = ue.per_tensor(ScaleDtype.F32), ue
+    tq = QTensorOps.quantize_dynamic(FloatOps.float_from_data(x, dev), two)
+    direct = FloatOps.float_into_data(QTensorOps.dequantize(tq))
+    blob = QTensorOps.q_into_data(tq)
+    assert blob.bytes.size == 256 + 8 + 4
+    assert FloatOps.float_into_data(QTensorOps.dequantize(QTensorOps.q_from_data(blob, dev))).tobytes() == direct.tobytes()
+
+    def error(t, scheme):
+        d = FloatOps.float_into_data(QTensorOps.dequantize(QTensorOps.quantize_dynamic(FloatOps.float_from_data(t, dev), scheme)))
+        return np.abs(t - d).sum() / np.abs(t).sum()
+
+    big = (np.arange(-128, 128, dtype=np.float32) / np.float32(128)).reshape(16, 16)
+    small = (big * np.float32(0.02)).astype(np.float32)
+    big_error, small_error = error(big, two), error(small, two)
+    assert abs(small_error - big_error) / big_error < 0.2
+    assert error(small, one) > small_error * 2.0
     # (the input whose largest relative scale lands one f32 step above 65504 before it is stored)
     big = (np.arange(-128, 128, dtype=np.float32) / np.float32(128)).reshape(16, 16)
     tb = QTensorOps.quantize_dynamic(FloatOps.float_from_data(big, dev), scheme)

@@ -533,3 +533,82 @@ def test_scale_dtype_accuracy_as_the_reference_measures_it():
     exact = rel_err(small, co.dequantize(q, sch, s))
     q2, _, _, eff = co.quantize_dynamic_two_level(small, sch, co.SCALE_F16)
     assert abs(rel_err(small, co.dequantize(q2, sch, eff)) - exact) / exact < 0.20
+
+
+def test_ue4m3_scales():
+    """The one-byte scale dtype: all 127 values of the non-negative half of e4m3 are fixed points of
+    scale_to_dtype, the f32 just above one goes to the next, the one just below the next stays
+    there; C (arithmetic) and numpy (table search) agree on 20 000 scales over 8 decades; the codec
+    maps value i to byte i; and the reference's layout test as it stands
+    (crates/burn-std/src/tensor/quantization.rs:659-684: 8 values + 2 one-byte block scales + f32)."""
+    vals = no.ue4m3_values().astype(np.float32)
+    assert vals.size == 127 and vals[-1] == 448 and vals[1] == 2.0 ** -9 and vals[8] == 2.0 ** -6
+    assert (co.scale_to_dtype(vals, co.SCALE_UE4M3) == vals).all()
+    assert (co.scale_to_dtype(np.nextafter(vals[:-1], np.float32(np.inf)), co.SCALE_UE4M3) == vals[1:]).all()
+    assert (co.scale_to_dtype(np.nextafter(vals[1:], np.float32(0)), co.SCALE_UE4M3) == vals[1:]).all()
+    r = np.exp(np.random.default_rng(0).uniform(np.log(1e-5), np.log(1000), 20000)).astype(np.float32)
+    up = co.scale_to_dtype(r, co.SCALE_UE4M3)
+    assert (up == no.scale_to_dtype(r, "UE4M3")).all() and (up[r <= 448] >= r[r <= 448]).all() and up.max() == 448
+    enc = co.encode_scales(vals, co.SCALE_UE4M3)
+    assert enc.tolist() == list(range(0x7F)) and (co.decode_scales(enc, co.SCALE_UE4M3) == vals).all()
+    assert (ba_f32_from_e4m3(enc) == vals).all()
+    values = np.int8([0, 25, 51, 76, 102, 127, -128, -1])
+    blob = co.encode_two_level(values, co.Scheme.make(co.Q8S, [4], co.STORE_NATIVE), np.float32([0.5, 0.125]),
+                               np.float32(3.0), co.SCALE_UE4M3)
+    assert blob.size == 8 + 2 + 4 and blob[8:10].tolist() == [0x30, 0x20] and blob[10:].view(np.float32)[0] == 3.0
+
+
+def ba_f32_from_e4m3(bits):
+    from burn_amd.ops import f32_from_e4m3_bits
+    return f32_from_e4m3_bits(bits)
+
+
+def test_ue4m3_behaviour_the_reference_asserts():
+    """Inequalities from the reference's own tests, on their inputs, which a wrong rounding direction,
+    a flush of small scales or a missing saturation would break: scheme.rs:50-90 (the largest relative
+    scale sits on 448, relative x global gives the one-level scales back), accuracy.rs:88-139
+    (one-level ue4m3 more than doubles the error at std 0.02; at std 1 it costs something, under 30 %),
+    ops/quantize.rs:238-290 (two-level error independent of magnitude, one-level degrades)."""
+    lo, hi = np.float32([-1.8, -0.5, 0.01, -0.04]), np.float32([0.5, 1.8, 0.04, -0.01])
+    one_level = co.compute_q_params(lo, hi, co.Q8S)
+    rel, g = co.normalize_scales(one_level, co.SCALE_UE4M3)
+    assert burn_approx_eq(rel.max(), 448.0, 0.005, 1e-5).all() and burn_approx_eq(rel * g, one_level, 0.005, 1e-5).all()
+
+    def normal_samples(n, std):
+        state, out = 0x2545F4914F6CDD1D, []
+        for _ in range(n):
+            u = []
+            for _ in range(2):
+                state = (state * 6364136223846793005 + 1442695040888963407) & 0xFFFFFFFFFFFFFFFF
+                u.append((np.float32(state >> 40) + np.float32(0.5)) / np.float32(1 << 24))
+            out.append(np.sqrt(np.float32(-2.0) * np.log(u[0])) * np.cos(np.float32(2 * np.pi) * u[1]) * np.float32(std))
+        return np.float32(out).reshape(64, 64)
+
+    def rel_err(x, d):
+        return np.sqrt(((x.astype(np.float64) - d) ** 2).sum()) / np.sqrt((x.astype(np.float64) ** 2).sum())
+
+    sch = co.Scheme.make(co.Q8S, [32], co.STORE_NATIVE)
+
+    def one_level_error(x, dtype):
+        _, s = co.quantize_dynamic(x, sch)
+        s = co.scale_to_dtype(s, dtype)
+        return rel_err(x, co.dequantize(co.quantize(x, sch, s), sch, s))
+
+    small, unit = normal_samples(64 * 64, 0.02), normal_samples(64 * 64, 1.0)
+    assert one_level_error(small, co.SCALE_UE4M3) > 2.0 * one_level_error(small, co.SCALE_F32)
+    f32_err, ue_err = one_level_error(unit, co.SCALE_F32), one_level_error(unit, co.SCALE_UE4M3)
+    assert f32_err < ue_err < 1.3 * f32_err
+
+    sch2 = co.Scheme.make(co.Q8S, [2, 16], co.STORE_NATIVE)
+    big = (np.arange(-128, 128, dtype=np.float32) / np.float32(128)).reshape(16, 16)
+    tiny = (big * np.float32(0.02)).astype(np.float32)
+
+    def two_level_error(t):
+        q, _, _, eff = co.quantize_dynamic_two_level(t, sch2, co.SCALE_UE4M3)
+        return np.abs(t - co.dequantize(q, sch2, eff)).sum() / np.abs(t).sum()
+
+    assert abs(two_level_error(tiny) - two_level_error(big)) / two_level_error(big) < 0.2
+    _, s = co.quantize_dynamic(tiny, sch2)
+    s = co.scale_to_dtype(s, co.SCALE_UE4M3)
+    one = np.abs(tiny - co.dequantize(co.quantize(tiny, sch2, s), sch2, s)).sum() / np.abs(tiny).sum()
+    assert one > 2.0 * two_level_error(tiny)
