@@ -561,7 +561,7 @@ size_t bqo_scale_size(int dtype) { return dtype == BQO_SCALE_F32 ? 4 : (dtype ==
  * above the smallest normal f32; every block scale is divided by it. One f32 operation per step,
  * as the tensor ops there (float_max, float_div_scalar, float_clamp_min, float_div). Returns the
  * per-tensor scale, or NaN for a block dtype the reference refuses (its largest value must not
- * exceed f16's: of f32 / f16 / bf16 that leaves f16, largest value 65504). */
+ * exceed f16's: f16, largest value 65504, and ue4m3, largest value 448). */
 float bqo_normalize_scales(float* scales, size_t n, int block_dtype) {
   if (block_dtype != BQO_SCALE_F16 && block_dtype != BQO_SCALE_UE4M3) return NAN;
   const float dtype_max = block_dtype == BQO_SCALE_F16 ? 65504.0f : 448.0f;

@@ -60,8 +60,8 @@
  *                        trip reproduces the dequantized values exactly, they are within 1e-2 of
  *                        the input, and the error does not track the weights' magnitude). The
  *                        largest value of the block dtype is f16's by the reference's own assert
- *                        (scheme.rs:115-118); UE4M3 blocks are not implemented. The quotient
- *                        top / (top / 65504) is 65504 or one f32 step above it, so this path takes
+ *                        (scheme.rs:115-118), ue4m3's is 448 (its bit pattern 0x7E). The quotient
+ *                        top / (top / dtype_max) is dtype_max or one f32 step above it, so this path takes
  *                        the saturating branch of bqo_scale_to_dtype about half of the time (PARITY
  *                        UNPINNED, see there). The reference's own two-level tests (ue4m3, same
  *                        arithmetic against 448) only pass if that branch saturates: on their input
