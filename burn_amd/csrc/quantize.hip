@@ -35,6 +35,9 @@ namespace {
 #ifndef BQ_ABSMAX_NT
 #define BQ_ABSMAX_NT 0
 #endif
+#ifndef BQ_QUANT_QUAD_STORE
+#define BQ_QUANT_QUAD_STORE 1
+#endif
 #ifndef BQ_QUANT_NT_STORE
 #define BQ_QUANT_NT_STORE 1
 #endif
@@ -118,6 +121,31 @@ constexpr int kBlockThreads = BQ_BLOCK_THREADS;      // run-block kernel
 constexpr int kBlockUnroll = BQ_BLOCK_UNROLL;
 constexpr int kTensorUnroll = BQ_TENSOR_UNROLL;      // per-tensor second pass
 
+// Lane 4j + i of a workgroup of T threads holds words chunk + T u + 4j + i, u = 0..3. A 4 x 4
+// transpose inside each quad of lanes (two rounds of DPP swaps) leaves lane 4j + i with the four
+// consecutive words chunk + T i + 4j + {0..3}: one 16-byte store per lane instead of four 4-byte
+// ones (1 % on the [8192, 8192] block quantize).
+template <int T>
+__device__ __forceinline__ void store_words_quad(uint32_t (&packed)[4], size_t chunk, uint32_t* __restrict__ out) {
+  const bool b0 = threadIdx.x & 1, b1 = threadIdx.x & 2;
+  auto swap1 = [](uint32_t v) { return static_cast<uint32_t>(__builtin_amdgcn_update_dpp(0, static_cast<int>(v), 0xB1, 0xF, 0xF, false)); };
+  auto swap2 = [](uint32_t v) { return static_cast<uint32_t>(__builtin_amdgcn_update_dpp(0, static_cast<int>(v), 0x4E, 0xF, 0xF, false)); };
+#pragma unroll
+  for (int p = 0; p < 4; p += 2) {   // round 1: lanes i and i ^ 1 exchange across registers p, p + 1
+    const uint32_t got = swap1(b0 ? packed[p] : packed[p + 1]);
+    if (b0) packed[p] = got; else packed[p + 1] = got;
+  }
+#pragma unroll
+  for (int p = 0; p < 2; ++p) {      // round 2: lanes i and i ^ 2 exchange across registers p, p + 2
+    const uint32_t got = swap2(b1 ? packed[p] : packed[p + 2]);
+    if (b1) packed[p] = got; else packed[p + 2] = got;
+  }
+  const size_t at = chunk + static_cast<size_t>(T) * (threadIdx.x & 3) + (threadIdx.x & ~3u);
+  const vuint4 v = {packed[0], packed[1], packed[2], packed[3]};
+  if (BQ_QUANT_NT_STORE) __builtin_nontemporal_store(v, reinterpret_cast<vuint4*>(out + at));
+  else *reinterpret_cast<vuint4*>(out + at) = v;
+}
+
 template <int VPL, int LANES, bool DYNAMIC>
 __global__ void __launch_bounds__(kBlockThreads)
 quantize_block_kernel(const float* __restrict__ x, size_t words, uint32_t* __restrict__ out,
@@ -126,6 +154,8 @@ quantize_block_kernel(const float* __restrict__ x, size_t words, uint32_t* __res
   constexpr int QMAX = (VPL == 4) ? 127 : 7;
   constexpr float SPAN = 2.0f * QMAX;
   const size_t base = static_cast<size_t>(blockIdx.x) * (kBlockThreads * U) + threadIdx.x;
+  constexpr bool kQuadStore = BQ_QUANT_QUAD_STORE && U == 4;
+  uint32_t packed[U];
   Vals<VPL> a[U];
 #pragma unroll
   for (int u = 0; u < U; ++u) {
@@ -162,7 +192,22 @@ quantize_block_kernel(const float* __restrict__ x, size_t words, uint32_t* __res
     }
     if (w < words) {
       if (DYNAMIC && (w & (LANES - 1)) == 0) scales_out[w / LANES] = s;
-      if (BQ_QUANT_NT_STORE) __builtin_nontemporal_store(word, out + w); else out[w] = word;
+      if (!kQuadStore) {
+        if (BQ_QUANT_NT_STORE) __builtin_nontemporal_store(word, out + w); else out[w] = word;
+      }
+    }
+    if (kQuadStore) packed[u] = word;
+  }
+  if (kQuadStore) {
+    const size_t chunk = static_cast<size_t>(blockIdx.x) * (kBlockThreads * U);
+    if (chunk + kBlockThreads * U <= words && (reinterpret_cast<uintptr_t>(out) & 15u) == 0) {
+      store_words_quad<kBlockThreads>(reinterpret_cast<uint32_t (&)[4]>(packed), chunk, out);
+    } else {
+#pragma unroll
+      for (int u = 0; u < U; ++u) {
+        const size_t w = base + static_cast<size_t>(u) * kBlockThreads;
+        if (w < words) out[w] = packed[u];
+      }
     }
   }
 }
@@ -281,15 +326,24 @@ quantize_tensor_kernel(const float* __restrict__ x, size_t n, const float* __res
   const float s = valid_scale(s_stored);
   const bool fast = recip_path_ok(s);
   const float r = recip_exact(s);
+  constexpr bool kQuadStore = BQ_QUANT_QUAD_STORE && U == 4;
+  const size_t chunk = static_cast<size_t>(blockIdx.x) * (kThreads * U);
+  // (out is the values region of a tensor or a caller's buffer: 16-byte stores need it aligned)
+  const bool quad = kQuadStore && chunk + kThreads * U <= words && (reinterpret_cast<uintptr_t>(out) & 15u) == 0;
+  uint32_t packed[U];
 #pragma unroll
   for (int u = 0; u < U; ++u) {
     const size_t w = base + static_cast<size_t>(u) * kThreads;
+    packed[u] = 0u;
     if (w < words)
     {
-      const uint32_t word = fast ? quantize_pack_recip<VPL, true>(a[u], s, r) : quantize_pack_div<VPL>(a[u], s);
-      if (BQ_QUANT_NT_STORE) __builtin_nontemporal_store(word, out + w); else out[w] = word;
+      packed[u] = fast ? quantize_pack_recip<VPL, true>(a[u], s, r) : quantize_pack_div<VPL>(a[u], s);
+      if (!quad) {
+        if (BQ_QUANT_NT_STORE) __builtin_nontemporal_store(packed[u], out + w); else out[w] = packed[u];
+      }
     }
   }
+  if (quad) store_words_quad<kThreads>(reinterpret_cast<uint32_t (&)[4]>(packed), chunk, out);
   // native i8 store with n % 4 != 0: the last 1..3 values, one byte each
   if (VPL == 4 && blockIdx.x == 0 && threadIdx.x == 0) {
     int8_t* bytes = reinterpret_cast<int8_t*>(out);
