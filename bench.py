@@ -477,6 +477,150 @@ def run_c5(ba, dev, steps, warmup, cpu):
 
 # ------------------------------------------------------------------------------ CPU baseline
 
+def run_next(ba, dev, steps, warmup, cpu):
+    """The callers and formats either side of the hot path, each gated against the oracle before
+    its figure is kept: the quantized Linear with its bias, narrow and two-level scale dtypes,
+    layout ops on packed tensors, ternary weights, and a burnpack file loaded to the device."""
+    import tempfile
+    from burn_amd import (FloatOps, QTensorOps, ModuleOps, QuantScheme, QuantValue, QuantStore, ScaleDtype,
+                          PackWriter, PackReader, TensorData)
+    from oracle import c_oracle as co
+    from oracle import np_oracle as no
+    out = {"timing": "HIP graphs over distinct tensors; ms per call"}
+    rng = np.random.default_rng(0xF0)
+
+    # ---- quantized Linear: the bias rides in the product's epilogue ------------------------------
+    k, n = 4096, 14336
+    w0 = quantized_weight(ba, dev, 0xC4, (k, n), QuantValue.Q8S)
+    blob = QTensorOps.q_into_data(w0)
+    ws = [w0] + [QTensorOps.q_from_data(blob, dev) for _ in range(15)]
+    values, scales = blob.split()
+    bias_h = rng.standard_normal(n, dtype=np.float32)
+    bias = FloatOps.float_from_data(bias_h, dev)
+    cols = np.arange(0, n, 37)
+    wd = unpack_columns(values, scales, k, n, cols, q4=False)
+    lin = {}
+    for m in (1, 16):
+        xh = rng.standard_normal((m, k), dtype=np.float32)
+        x = FloatOps.float_from_data(xh, dev)
+        got = FloatOps.float_into_data(ModuleOps.linear(x, ws[3], bias))[:, cols]
+        matmul_gate(f"linear M={m}", got, xh.astype(np.float64) @ wd + bias_h[cols].astype(np.float64))
+        t_lin = graph_ms(dev, lambda: [ModuleOps.linear(x, wq, bias) for wq in ws], 16, steps, warmup)
+        t_mm = graph_ms(dev, lambda: [QTensorOps.q_matmul(x, wq) for wq in ws], 16, steps, warmup)
+        lin[f"M={m}"] = {"ms": t_lin, "ms_without_bias": t_mm, "GB/s": (k * n + 4 * k * n // 32) / t_lin / 1e6}
+    out["linear"] = {"workload": "x[M,4096] f32 x Q8S block-32 [4096,14336] + bias[14336] -> f32 (C4's weight)",
+                     "parity": "vs float64 on every 37th column, rel 1e-2 and burn's elementwise rule", **lin}
+    del ws, w0, blob, values, scales
+    dev.trim()
+
+    # ---- scale dtypes: quantize_dynamic + dequantize of C2's tensor ------------------------------
+    rows = 8192
+    nel = rows * 8192
+    host = normal_f32(0xC2, (rows, 8192), outliers=True)
+    xs = [FloatOps.float_from_data(np.roll(host, i * 977, axis=0), dev) for i in range(5)]
+    small = np.ascontiguousarray(host[:256])
+    codes = {ScaleDtype.F16: co.SCALE_F16, ScaleDtype.BF16: co.SCALE_BF16, ScaleDtype.UE4M3: co.SCALE_UE4M3}
+    osch = co.Scheme.make(co.Q8S, [32], co.STORE_PACKED_U32)
+    sd = {}
+    for name, sdt, two in (("f16", ScaleDtype.F16, False), ("bf16", ScaleDtype.BF16, False), ("ue4m3", ScaleDtype.UE4M3, False),
+                           ("f16 under f32", ScaleDtype.F16, True), ("ue4m3 under f32", ScaleDtype.UE4M3, True)):
+        scheme = QuantScheme().per_block((32,), sdt)
+        if two:
+            scheme = scheme.per_tensor(ScaleDtype.F32)
+        tq = QTensorOps.quantize_dynamic(FloatOps.float_from_data(small, dev), scheme)
+        if two:
+            q_ref, stored, g, eff = co.quantize_dynamic_two_level(small, osch, codes[sdt])
+            want = co.encode_two_level(q_ref, osch, stored, g, codes[sdt])
+        else:
+            lo, hi = co.compute_range(small, osch)
+            eff = co.scale_to_dtype(co.compute_q_params(lo, hi, osch.value), codes[sdt])
+            q_ref = co.quantize(small, osch, eff)
+            want = co.encode_with_scale_dtype(q_ref, osch, eff, codes[sdt])
+        if QTensorOps.q_into_data(tq).bytes.tobytes() != want.tobytes():
+            raise ParityError(f"{name} scales: the blob differs from the CPU oracle's")
+        if FloatOps.float_into_data(QTensorOps.dequantize(tq)).tobytes() != co.dequantize(q_ref, osch, eff).tobytes():
+            raise ParityError(f"{name} scales: dequantize differs from the CPU oracle")
+        t_q = graph_ms(dev, lambda: [QTensorOps.quantize_dynamic(xs[i % 5], scheme) for i in range(10)], 10, steps, warmup)
+        qs = [QTensorOps.quantize_dynamic(xs[i % 5], scheme) for i in range(16)]
+        t_d = graph_ms(dev, lambda: [QTensorOps.dequantize(q) for q in qs], 16, steps, warmup)
+        del qs
+        b = 4 * nel + nel + sdt.size() * nel // 32 + (4 if two else 0)
+        sd[name] = {"quantize_dynamic": {"ms": t_q, "GB/s": b / t_q / 1e6, "frac_hbm": b / t_q / 1e6 / HBM_PEAK_GBS},
+                    "dequantize": {"ms": t_d, "GB/s": b / t_d / 1e6, "frac_hbm": b / t_d / 1e6 / HBM_PEAK_GBS}, "bytes": b}
+        dev.trim()
+    out["scale_dtypes"] = {"workload": "C2's tensor, Q8S block-32 PackedU32, block scales stored as f16 / bf16 / ue4m3, alone or "
+                                       "relative to an f32 per-tensor scale (two launches more: the largest scale, the split)",
+                           "parity": "blob and dequantized floats bit-exact vs CPU oracle on a 256-row tensor of the same data", **sd}
+
+    # ---- layout ops on a packed tensor -------------------------------------------------------------
+    scheme = QuantScheme().per_block((32,))
+    tq_small = QTensorOps.quantize_dynamic(FloatOps.float_from_data(small, dev), scheme)
+    q_ref, s_ref = co.quantize_dynamic(small, osch)
+    tr = QTensorOps.q_into_data(QTensorOps.q_swap_dims(tq_small, 0, 1))
+    tv, ts = tr.split()
+    if no.unpack_u32(tv.view(np.uint32), tr.shape, "Q8S").tobytes() != np.ascontiguousarray(q_ref.T).tobytes() or \
+            ts.reshape(-1).tobytes() != np.ascontiguousarray(s_ref.reshape(256, 256).T).tobytes():
+        raise ParityError("swap_dims of a packed block-quantized tensor differs from the oracle's transpose")
+    qs = [QTensorOps.quantize_dynamic(xs[i % 5], scheme) for i in range(8)]
+    t_t = graph_ms(dev, lambda: [QTensorOps.q_swap_dims(q, 0, 1) for q in qs], 8, steps, warmup)
+    b = 2 * (nel + 4 * nel // 32)
+    out["layout"] = {"workload": "q_swap_dims(0, 1) of a Q8S block-32 PackedU32 [8192,8192] tensor: values repacked along "
+                                 "the new last dim, scales moved with their blocks",
+                     "parity": "values and scales bit-exact vs the transposed oracle tensor, 256 x 8192",
+                     "swap_dims": {"ms": t_t, "GB/s": b / t_t / 1e6, "frac_hbm": b / t_t / 1e6 / HBM_PEAK_GBS, "bytes": b}}
+    del qs, xs
+    dev.trim()
+
+    # ---- ternary weights ---------------------------------------------------------------------------
+    wt = normal_f32(0xF4, (k, n), 0.02)
+    tsch = QuantScheme(value=QuantValue.Q2S)
+    tws = [QTensorOps.quantize_dynamic(FloatOps.float_from_data(wt, dev), tsch) for _ in range(8)]
+    tblob = QTensorOps.q_into_data(tws[0])
+    tvals, tscale = tblob.split()
+    q_t = no.unpack_u32(tvals.view(np.uint32), (k, n), "Q2S")
+    tern = {}
+    for m in (1, 16):
+        xh = rng.standard_normal((m, k), dtype=np.float32)
+        x = FloatOps.float_from_data(xh, dev)
+        got = FloatOps.float_into_data(QTensorOps.q_matmul(x, tws[1]))
+        ref = (xh.astype(np.float64) @ q_t[:, cols].astype(np.float64)) * np.float64(tscale.reshape(-1)[0])
+        matmul_gate(f"ternary M={m}", got[:, cols], ref)
+        t = graph_ms(dev, lambda: [QTensorOps.q_matmul(x, wq) for wq in tws], 8, steps, warmup)
+        tb = k * n // 4 + 4
+        tern[f"M={m}"] = {"ms": t, "GB/s": tb / t / 1e6, "frac_hbm": tb / t / 1e6 / HBM_PEAK_GBS}
+    out["ternary"] = {"workload": "x[M,4096] f32 x Q2S per-tensor PackedU32 [4096,14336] (16 values per word) -> f32",
+                      "parity": "vs float64 on every 37th column, rel 1e-2 and burn's elementwise rule", **tern}
+    del tws
+    dev.trim()
+
+    # ---- a burnpack file to the device -------------------------------------------------------------
+    w3 = quantized_weight(ba, dev, 0xC3, (14336, 4096), QuantValue.Q4S)
+    want = QTensorOps.q_into_data(w3).bytes.tobytes()
+    wr = PackWriter()
+    wr.add_tensor("mlp.up_proj.weight", w3)
+    with tempfile.TemporaryDirectory() as tmp:
+        path = os.path.join(tmp, "c3.bpk")
+        wr.write_to_file(path)
+        size = os.path.getsize(path)
+        best = None
+        for _ in range(3):
+            t0 = time.perf_counter()
+            rd = PackReader(path)
+            t = rd.load("mlp.up_proj.weight", dev)
+            dev.sync()
+            dt = time.perf_counter() - t0
+            rd.close()
+            best = dt if best is None else min(best, dt)
+        if QTensorOps.q_into_data(t).bytes.tobytes() != want:
+            raise ParityError("the tensor loaded from the burnpack file differs from the one written")
+    out["burnpack"] = {"workload": "C3's weight (Q4S block-32 [14336,4096]) written to a burnpack file and loaded back to the "
+                                   "device: open, parse, one host-to-device copy of values || scales",
+                       "parity": "blob of the loaded tensor byte-identical to the written one's",
+                       "file_bytes": size, "load_ms": best * 1e3, "GB/s": size / best / 1e9,
+                       "note": "host path (page cache + PCIe), not an HBM figure"}
+    return out
+
+
 def cpu_baseline_c2(passes=5):
     """The oracle (port of burn-ndarray's serial loops), one thread, on the whole C2 tensor,
     `passes` times over (about 10 s of CPU work)."""
@@ -509,7 +653,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--no-others", action="store_true", help="skip the C1/C3/C4/C5 side measurements")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline legs")
-    ap.add_argument("--only", default="", help="comma list of side configs to run (c1,c3,c4,c5)")
+    ap.add_argument("--only", default="", help="comma list of side configs to run (c1,c3,c4,c5,next)")
     ap.add_argument("--c5-n", type=int, default=C5_N, help="weight columns of the C5 side measurement (default: C5's 14336)")
     args = ap.parse_args()
     C5_N = args.c5_n
@@ -562,7 +706,7 @@ def main():
     if not args.no_others:
         only = [s for s in args.only.split(",") if s]
         others = {}
-        for key, fn in (("c1", run_c1), ("c3", run_c3), ("c4", run_c4), ("c5", run_c5)):
+        for key, fn in (("c1", run_c1), ("c3", run_c3), ("c4", run_c4), ("c5", run_c5), ("next", run_next)):
             if only and key not in only:
                 continue
             log(f"{key} ...")

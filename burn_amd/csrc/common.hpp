@@ -133,6 +133,12 @@ bq_status launch_round_scales(const float* src, float* dst, size_t n, int scale_
 // Two-level schemes. split: `scales` holds the f32 block scales of a quantize_dynamic and `cells` the
 // partial maxima over them (bqk_absmax_f32); on return scales[i] = global * stored[i], the scale
 // the kernels use. times_global: the same product from a stored pair.
+// Two-level quantize_dynamic in one pass over x: the per-tensor scale from the absmax cells of the whole
+// tensor, then the run-block kernel that splits every block scale against it as it computes it.
+bq_status launch_two_level_global(const uint32_t* cells, int value, int scale_dtype, float* global_out, hipStream_t stream);
+bq_status launch_quantize_run_block_two_level(const float* x, size_t n, int block, const float* global, float* stored_out,
+                                              float* scales_out, int value, int store, void* values, int scale_dtype,
+                                              hipStream_t stream);
 bq_status launch_two_level_split(float* scales, size_t n, const uint32_t* cells, int scale_dtype, float* global_out,
                                  float* stored, hipStream_t stream);
 bq_status launch_scales_times_global(const float* stored, const float* global, size_t n, float* scales, hipStream_t stream);

@@ -1,9 +1,10 @@
 // Layout ops on quantized tensors for gfx950: q_permute / q_swap_dims / q_flip
 // (crates/burn-ndarray/src/ops/qtensor.rs:301-347). The reference permutes the values and, for
 // block schemes, the scales with their blocks (scheme.permute_block_dims); tensors here are
-// always dense row-major, so the result is materialised by a gather: one thread per output word
-// (4 x i8 or 8 x i4 along the new last dim), each element fetched from its source position.
-// Complete rather than fast: these are set-up operations (a transposed weight), not the hot loop.
+// always dense row-major, so the result is materialised: by a tiled transpose when 8-bit values
+// swap their last two dims (a transposed weight, the usual case), else by a gather, one thread per
+// output word (4 x i8, 8 x i4 or 16 x i2 along the new last dim), each element fetched from its
+// source position. These are set-up operations, not the hot loop.
 #include "common.hpp"
 #include "device_math.hpp"
 
@@ -18,19 +19,22 @@ struct GatherDims {
   uint32_t flip[BQ_MAX_RANK];    // output dim d runs backwards over its source dim
 };
 
-__device__ __forceinline__ size_t source_index(const GatherDims& d, size_t e) {
-  size_t idx = 0;
+// I: uint32_t when every element index fits 32 bits (a 64-bit division costs several times a
+// 32-bit one, and there is one per dim and element).
+template <typename I>
+__device__ __forceinline__ size_t source_index(const GatherDims& d, I e) {
+  I idx = 0;
   for (int a = d.rank - 1; a >= 0; --a) {
-    size_t c = e % d.shape[a];
-    e /= d.shape[a];
-    if (d.flip[a]) c = d.shape[a] - 1 - c;
-    idx += c * d.stride[a];
+    I c = e % static_cast<I>(d.shape[a]);
+    e /= static_cast<I>(d.shape[a]);
+    if (d.flip[a]) c = static_cast<I>(d.shape[a]) - 1 - c;
+    idx += c * static_cast<I>(d.stride[a]);
   }
   return idx;
 }
 
 // BITS-wide fields; `native`: one i8 per element (n need not be a multiple of 4), else u32 words.
-template <int BITS>
+template <int BITS, typename I>
 __global__ void __launch_bounds__(256)
 q_gather_kernel(const uint32_t* __restrict__ src, uint32_t* __restrict__ dst, size_t n, GatherDims d, bool native) {
   constexpr int EPW = 32 / BITS;
@@ -42,7 +46,7 @@ q_gather_kernel(const uint32_t* __restrict__ src, uint32_t* __restrict__ dst, si
   for (int j = 0; j < EPW; ++j) {
     const size_t e = e0 + j;
     if (e >= n) break;
-    const size_t idx = source_index(d, e);
+    const size_t idx = source_index<I>(d, static_cast<I>(e));
     uint32_t v;
     if (BITS == 8)
       v = reinterpret_cast<const uint8_t*>(src)[idx];
@@ -57,10 +61,58 @@ q_gather_kernel(const uint32_t* __restrict__ src, uint32_t* __restrict__ dst, si
   }
 }
 
+template <typename I>
 __global__ void __launch_bounds__(256)
 f32_gather_kernel(const float* __restrict__ src, float* __restrict__ dst, size_t n, GatherDims d) {
   const size_t e = static_cast<size_t>(blockIdx.x) * 256 + threadIdx.x;
-  if (e < n) dst[e] = src[source_index(d, e)];
+  if (e < n) dst[e] = src[source_index<I>(d, static_cast<I>(e))];
+}
+
+// 8-bit values, last two dims swapped: dst[b][c][r] = src[b][r][c], R and C multiples of 4. A
+// workgroup moves a tile of 128 x 128 bytes. A thread loads the same word column of 4 consecutive
+// rows, transposes the 4 x 4 bytes in registers (8 byte permutes) and writes the 4 resulting words
+// -- 4 output rows, one word each -- to LDS; the tile leaves as whole 128-byte output rows. LDS row
+// of output row 4 w + j is 32 j + w and rows are 33 words apart, so both the writes (w varies over
+// the lanes) and the reads (the word index does) are spread over all banks.
+constexpr int kTile = 128;
+constexpr int kTileWords = kTile / 4;
+
+__global__ void __launch_bounds__(256)
+q8_transpose_kernel(const uint32_t* __restrict__ src, uint32_t* __restrict__ dst, uint32_t R, uint32_t C) {
+  __shared__ uint32_t tile[kTile][kTileWords + 1];
+  const size_t plane = static_cast<size_t>(R) * C / 4;  // words per batch entry
+  src += plane * blockIdx.z;
+  dst += plane * blockIdx.z;
+  const uint32_t r0 = blockIdx.y * kTile, c0 = blockIdx.x * kTile;
+  const uint32_t cw = C / 4, rw = R / 4;
+  const uint32_t w = threadIdx.x % kTileWords, q0 = threadIdx.x / kTileWords;  // word column; first row quad (of 8 per pass)
+#pragma unroll
+  for (uint32_t pass = 0; pass < 4; ++pass) {
+    const uint32_t g = q0 + 8 * pass;  // row quad of the tile: rows 4 g .. 4 g + 3
+    uint32_t in[4];
+#pragma unroll
+    for (uint32_t i = 0; i < 4; ++i) {
+      const uint32_t r = r0 + 4 * g + i, c = c0 / 4 + w;
+      in[i] = (r < R && c < cw) ? __builtin_nontemporal_load(src + static_cast<size_t>(r) * cw + c) : 0u;
+    }
+    // bytes (row i, column j) -> word j holds rows 0..3 of column j, low byte first
+    const uint32_t t0 = __builtin_amdgcn_perm(in[1], in[0], 0x05010400u), t1 = __builtin_amdgcn_perm(in[1], in[0], 0x07030602u);
+    const uint32_t t2 = __builtin_amdgcn_perm(in[3], in[2], 0x05010400u), t3 = __builtin_amdgcn_perm(in[3], in[2], 0x07030602u);
+    tile[0 * kTileWords + w][g] = __builtin_amdgcn_perm(t2, t0, 0x05040100u);
+    tile[1 * kTileWords + w][g] = __builtin_amdgcn_perm(t2, t0, 0x07060302u);
+    tile[2 * kTileWords + w][g] = __builtin_amdgcn_perm(t3, t1, 0x05040100u);
+    tile[3 * kTileWords + w][g] = __builtin_amdgcn_perm(t3, t1, 0x07060302u);
+  }
+  __syncthreads();
+  // output row c0 + cc, words r0 / 4 + (0 .. 31): a wave writes two whole 128-byte rows per store
+  const uint32_t g = threadIdx.x % kTileWords;
+#pragma unroll
+  for (uint32_t pass = 0; pass < kTile / 8; ++pass) {
+    const uint32_t cc = threadIdx.x / kTileWords + 8 * pass;
+    const uint32_t c = c0 + cc, rq = r0 / 4 + g;
+    if (c < C && rq < rw)
+      __builtin_nontemporal_store(tile[(cc & 3u) * kTileWords + (cc >> 2)][g], dst + static_cast<size_t>(c) * rw + rq);
+  }
 }
 
 GatherDims make_dims(const size_t* src_shape, int rank, const int32_t* axes, const uint8_t* flip) {
@@ -89,19 +141,42 @@ bq_status launch_q_gather(const void* src, void* dst, const size_t* src_shape, i
   size_t n = 1;
   for (int a = 0; a < rank; ++a) n *= src_shape[a];
   if (n == 0) return BQ_OK;
+  // 8-bit values whose last two dims trade places (leading dims in place, nothing flipped), both
+  // in whole words: the tiled transpose
+  if (value == BQ_Q8S && rank >= 2 && axes[rank - 1] == rank - 2 && axes[rank - 2] == rank - 1) {
+    bool plain = true;
+    size_t batch = 1;
+    for (int a = 0; a < rank; ++a) plain = plain && !(flip && flip[a]);
+    for (int a = 0; a + 2 < rank; ++a) {
+      plain = plain && axes[a] == a;
+      batch *= src_shape[a];
+    }
+    const size_t rows = src_shape[rank - 2], cols = src_shape[rank - 1];
+    const size_t tr = (rows + kTile - 1) / kTile, tc = (cols + kTile - 1) / kTile;
+    if (plain && rows % 4 == 0 && cols % 4 == 0 && rows < 0x7FFFFFFFu && cols < 0x7FFFFFFFu && tr <= 65535 && batch <= 65535 &&
+        (reinterpret_cast<uintptr_t>(src) & 3u) == 0 && (reinterpret_cast<uintptr_t>(dst) & 3u) == 0) {
+      hipLaunchKernelGGL(q8_transpose_kernel, dim3(static_cast<unsigned>(tc), static_cast<unsigned>(tr), static_cast<unsigned>(batch)),
+                         dim3(256), 0, st, static_cast<const uint32_t*>(src), static_cast<uint32_t*>(dst),
+                         static_cast<uint32_t>(rows), static_cast<uint32_t>(cols));
+      BQ_HIP(hipGetLastError());
+      return BQ_OK;
+    }
+  }
   const GatherDims d = make_dims(src_shape, rank, axes, flip);
   const int epw = num_quants(value);
   const size_t units = (n + epw - 1) / epw;
+  if ((units + 255) / 256 > 0x7FFFFFFFu) BQ_FAIL(BQ_ERR_SIZE, "permute of %zu values exceeds the launch grid", n);
   dim3 grid(static_cast<unsigned>((units + 255) / 256)), tb(256);
-  if (value == BQ_Q8S)
-    hipLaunchKernelGGL(q_gather_kernel<8>, grid, tb, 0, st, static_cast<const uint32_t*>(src),
-                       static_cast<uint32_t*>(dst), n, d, native);
-  else if (value == BQ_Q4S)
-    hipLaunchKernelGGL(q_gather_kernel<4>, grid, tb, 0, st, static_cast<const uint32_t*>(src),
-                       static_cast<uint32_t*>(dst), n, d, false);
-  else
-    hipLaunchKernelGGL(q_gather_kernel<2>, grid, tb, 0, st, static_cast<const uint32_t*>(src),
-                       static_cast<uint32_t*>(dst), n, d, false);
+  const uint32_t* s32 = static_cast<const uint32_t*>(src);
+  uint32_t* d32 = static_cast<uint32_t*>(dst);
+  const bool small = n <= 0xFFFFFFFFull;
+#define BQ_GATHER(B, NATIVE)                                                                  \
+  if (small) hipLaunchKernelGGL((q_gather_kernel<B, uint32_t>), grid, tb, 0, st, s32, d32, n, d, NATIVE); \
+  else hipLaunchKernelGGL((q_gather_kernel<B, size_t>), grid, tb, 0, st, s32, d32, n, d, NATIVE)
+  if (value == BQ_Q8S) { BQ_GATHER(8, native); }
+  else if (value == BQ_Q4S) { BQ_GATHER(4, false); }
+  else { BQ_GATHER(2, false); }
+#undef BQ_GATHER
   BQ_HIP(hipGetLastError());
   return BQ_OK;
 }
@@ -113,7 +188,11 @@ bq_status launch_f32_gather(const float* src, float* dst, const size_t* src_shap
   for (int a = 0; a < rank; ++a) n *= src_shape[a];
   if (n == 0) return BQ_OK;
   const GatherDims d = make_dims(src_shape, rank, axes, flip);
-  hipLaunchKernelGGL(f32_gather_kernel, dim3(static_cast<unsigned>((n + 255) / 256)), dim3(256), 0, st, src, dst, n, d);
+  if ((n + 255) / 256 > 0x7FFFFFFFu) BQ_FAIL(BQ_ERR_SIZE, "permute of %zu scales exceeds the launch grid", n);
+  if (n <= 0xFFFFFFFFull)
+    hipLaunchKernelGGL(f32_gather_kernel<uint32_t>, dim3(static_cast<unsigned>((n + 255) / 256)), dim3(256), 0, st, src, dst, n, d);
+  else
+    hipLaunchKernelGGL(f32_gather_kernel<size_t>, dim3(static_cast<unsigned>((n + 255) / 256)), dim3(256), 0, st, src, dst, n, d);
   BQ_HIP(hipGetLastError());
   return BQ_OK;
 }

@@ -523,51 +523,81 @@ __global__ void bf16_to_f32_kernel(const uint16_t* __restrict__ src, size_t n, f
 // Ternary weights (Q2S: -1, 0, +1, 16 per word) times f32 activations, without a multiply in the
 // sum: +1 adds the activation, -1 subtracts it, anything else leaves the sum alone, and the
 // per-tensor scale multiplies the finished sum once -- crates/burn-ndarray/src/ops/qtensor.rs:431-517.
-// A lane owns one packed word column (16 outputs) and RM activation rows and walks k in ascending
-// order, which is the reference's order of additions: the results are the reference's bit for bit.
-template <int RM>
+// An output's additions are made in ascending k, the reference's order, by one lane: the results
+// are the reference's bit for bit, and the chain of K dependent additions is the kernel's time
+// (an add per k, plus the field's decode off the chain). A lane owns one output column and one
+// activation row (grid.y). The 16 lanes that share a packed word column load it for 16
+// consecutive rows, one row each, and hand the rows round by DPP row broadcast; kTernaryDepth such
+// loads are in flight per lane. The addend is built with bit operations -- x, its sign flipped
+// when the field's high bit is set, masked to +0 when its low bit is clear -- and sum + (+0) is
+// the sum itself here (a sum that starts at +0 never becomes -0), so a skipped field, an infinite
+// or a NaN activation included, leaves the sum alone as the reference's `match` does.
+constexpr int kTernaryDepth = 4;  // (8, 12, 16 measured the same: the chain of additions is the time)
+
+template <int J>
+__device__ __forceinline__ uint32_t ternary_row(uint32_t v) {  // the value lane J of this row of 16 lanes holds
+  return static_cast<uint32_t>(__builtin_amdgcn_update_dpp(0, static_cast<int>(v), 0x150 + J, 0xF, 0xF, true));
+}
+
 __global__ void __launch_bounds__(256)
 ternary_matmul_kernel(const float* __restrict__ x, const uint32_t* __restrict__ w, const float* __restrict__ scale,
-                      size_t M, size_t K, size_t NW, float* __restrict__ out) {
-  const size_t wc = static_cast<size_t>(blockIdx.x) * 256 + threadIdx.x;
-  const size_t m0 = static_cast<size_t>(blockIdx.y) * RM;
-  if (wc >= NW) return;
-  float acc[RM][16];
+                      size_t K, size_t NW, float* __restrict__ out) {
+  constexpr int D = kTernaryDepth;
+  const size_t N = NW * 16;
+  const size_t col = static_cast<size_t>(blockIdx.x) * 256 + threadIdx.x;
+  const bool active = col < N;  // (N is a multiple of 16: the 16 lanes of a word are active together)
+  const size_t wc = active ? col >> 4 : 0;
+  const unsigned j = threadIdx.x & 15u, shift = 2u * j;
+  const float* __restrict__ xr = x + static_cast<size_t>(blockIdx.y) * K;
+  auto fetch = [&](size_t k0) {
+    const size_t r = k0 + j;
+    return (active && r < K) ? w[r * NW + wc] : 0u;  // rows past the end: zero fields add nothing
+  };
+  uint32_t ring[D];
 #pragma unroll
-  for (int r = 0; r < RM; ++r)
+  for (int d = 0; d < D; ++d) ring[d] = fetch(16u * d);
+  float acc = 0.0f;
+  for (size_t k0 = 0; k0 < K; k0 += 16 * D) {
 #pragma unroll
-    for (int j = 0; j < 16; ++j) acc[r][j] = 0.0f;
-  for (size_t k = 0; k < K; ++k) {
-    const uint32_t word = w[k * NW + wc];
-#pragma unroll
-    for (int r = 0; r < RM; ++r) {
-      const float xv = m0 + r < M ? x[(m0 + r) * K + k] : 0.0f;
-#pragma unroll
-      for (int j = 0; j < 16; ++j) {
-        const uint32_t f = (word >> (2 * j)) & 3u;  // two's complement: 1 = +1, 3 = -1, 0 and 2 are skipped
-        acc[r][j] = f == 1u ? acc[r][j] + xv : (f == 3u ? acc[r][j] - xv : acc[r][j]);
-      }
+    for (int d = 0; d < D; ++d) {
+      const uint32_t cur = ring[d];
+      ring[d] = fetch(k0 + 16u * (d + D));
+      const size_t kb = k0 + 16u * d;
+      if (kb >= K) break;  // (uniform)
+      // rows kb .. kb + 15, in order; FULL: all of them exist (their activations are 16 contiguous
+      // scalar loads), else the tail of K, row by row
+#define BQ_TERNARY_STEP(JJ)                                                                          \
+  {                                                                                                  \
+    const uint32_t word = ternary_row<JJ>(cur);                                                      \
+    const uint32_t xb = __builtin_bit_cast(uint32_t, (full || kb + JJ < K) ? xr[kb + JJ] : 0.0f);    \
+    const uint32_t keep = static_cast<uint32_t>(__builtin_amdgcn_sbfe(static_cast<int>(word), shift, 1u));      /* +-1: all ones */ \
+    const uint32_t flip = static_cast<uint32_t>(__builtin_amdgcn_sbfe(static_cast<int>(word), shift + 1u, 1u)) & 0x80000000u; /* -1: the sign */ \
+    acc += __builtin_bit_cast(float, (xb ^ flip) & keep);                                            \
+  }
+      auto group = [&](auto FULL) {
+        constexpr bool full = decltype(FULL)::value;
+        BQ_TERNARY_STEP(0) BQ_TERNARY_STEP(1) BQ_TERNARY_STEP(2) BQ_TERNARY_STEP(3)
+        BQ_TERNARY_STEP(4) BQ_TERNARY_STEP(5) BQ_TERNARY_STEP(6) BQ_TERNARY_STEP(7)
+        BQ_TERNARY_STEP(8) BQ_TERNARY_STEP(9) BQ_TERNARY_STEP(10) BQ_TERNARY_STEP(11)
+        BQ_TERNARY_STEP(12) BQ_TERNARY_STEP(13) BQ_TERNARY_STEP(14) BQ_TERNARY_STEP(15)
+      };
+      if (kb + 16 <= K) group(std::true_type{}); else group(std::false_type{});
+#undef BQ_TERNARY_STEP
     }
   }
-  const float gamma = scale[0];
-  const size_t N = NW * 16;
-#pragma unroll
-  for (int r = 0; r < RM; ++r) {
-    if (m0 + r >= M) break;
-    vfloat4* dst = reinterpret_cast<vfloat4*>(out + (m0 + r) * N + wc * 16);
-#pragma unroll
-    for (int q = 0; q < 4; ++q)
-      dst[q] = vfloat4{acc[r][4 * q] * gamma, acc[r][4 * q + 1] * gamma, acc[r][4 * q + 2] * gamma, acc[r][4 * q + 3] * gamma};
-  }
+  if (active) out[static_cast<size_t>(blockIdx.y) * N + col] = acc * scale[0];
 }
 
 bq_status launch_ternary_matmul(const float* x, const uint32_t* w, const float* scale, size_t m, size_t k, size_t n,
                                 float* out, hipStream_t st) {
   if (m == 0 || n == 0) return BQ_OK;
   const size_t nw = n / 16;
-  dim3 grid(static_cast<unsigned>((nw + 255) / 256), static_cast<unsigned>((m + 3) / 4)), tb(256);
-  hipLaunchKernelGGL(ternary_matmul_kernel<4>, grid, tb, 0, st, x, w, scale, m, k, nw, out);
-  BQ_HIP(hipGetLastError());
+  for (size_t m0 = 0; m0 < m; m0 += 65535u) {  // (grid.y holds 65535 rows)
+    const size_t rows = std::min<size_t>(65535u, m - m0);
+    dim3 grid(static_cast<unsigned>((n + 255) / 256), static_cast<unsigned>(rows)), tb(256);
+    hipLaunchKernelGGL(ternary_matmul_kernel, grid, tb, 0, st, x + m0 * k, w, scale, k, nw, out + m0 * n);
+    BQ_HIP(hipGetLastError());
+  }
   return BQ_OK;
 }
 

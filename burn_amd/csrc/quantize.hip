@@ -146,10 +146,17 @@ __device__ __forceinline__ void store_words_quad(uint32_t (&packed)[4], size_t c
   else *reinterpret_cast<vuint4*>(out + at) = v;
 }
 
-template <int VPL, int LANES, bool DYNAMIC>
+// TWO (dynamic only): block scales relative to a per-tensor scale. `scales_in` then points at that
+// one f32 (global), `stored_out` receives a block's scale as it is stored, scale_to_dtype(s / global)
+// in the dtype `sdt`, and the block is quantized against global * that, which goes to `scales_out`
+// -- normalize_scales (crates/burn-backend/src/quantization/scheme.rs:106-134) and what
+// NdArray::quantize makes of its result, one IEEE operation per step as there.
+template <int VPL, int LANES, bool DYNAMIC, bool TWO = false>
 __global__ void __launch_bounds__(kBlockThreads)
 quantize_block_kernel(const float* __restrict__ x, size_t words, uint32_t* __restrict__ out,
-                      float* __restrict__ scales_out, const float* __restrict__ scales_in, int sdt) {
+                      float* __restrict__ scales_out, const float* __restrict__ scales_in, int sdt,
+                      float* __restrict__ stored_out = nullptr) {
+  static_assert(!TWO || DYNAMIC, "two-level scales are split where the block scales are computed");
   constexpr int U = kBlockUnroll;
   constexpr int QMAX = (VPL == 4) ? 127 : 7;
   constexpr float SPAN = 2.0f * QMAX;
@@ -174,7 +181,15 @@ quantize_block_kernel(const float* __restrict__ x, size_t words, uint32_t* __res
     const size_t w = base + static_cast<size_t>(u) * kBlockThreads;
     uint32_t word;
     float s;
-    if (DYNAMIC) {
+    float stored = 0.0f;
+    if (TWO) {
+      const float m = group_max<LANES>(absmax_vals<VPL>(a[u]));
+      const float one_level = absmax_fast_ok(m) ? scale_from_absmax_fast<QMAX>(m) : scale_from_absmax(m, SPAN);
+      const float global = scales_in[0];
+      stored = scale_round_up(one_level / global, sdt);
+      s = global * stored;
+      word = quantize_pack<VPL>(a[u], s);
+    } else if (DYNAMIC) {
       const float m = group_max<LANES>(absmax_vals<VPL>(a[u]));
       if (sdt != BQ_SCALE_F32) {  // f16 / bf16 scales: divide by the scale as it will be stored
         s = scale_round_up(absmax_fast_ok(m) ? scale_from_absmax_fast<QMAX>(m) : scale_from_absmax(m, SPAN), sdt);
@@ -192,6 +207,7 @@ quantize_block_kernel(const float* __restrict__ x, size_t words, uint32_t* __res
     }
     if (w < words) {
       if (DYNAMIC && (w & (LANES - 1)) == 0) scales_out[w / LANES] = s;
+      if (TWO && (w & (LANES - 1)) == 0) stored_out[w / LANES] = stored;
       if (!kQuadStore) {
         if (BQ_QUANT_NT_STORE) __builtin_nontemporal_store(word, out + w); else out[w] = word;
       }
@@ -440,16 +456,16 @@ inline unsigned grid_for(size_t items, unsigned cap) {
   return static_cast<unsigned>(g < cap ? g : cap);
 }
 
-template <int VPL, bool DYNAMIC>
+template <int VPL, bool DYNAMIC, bool TWO = false>
 bq_status launch_block(const float* x, size_t n, int block, uint32_t* out, float* scales_out,
-                       const float* scales_in, int sdt, hipStream_t st) {
+                       const float* scales_in, int sdt, hipStream_t st, float* stored_out = nullptr) {
   const size_t words = n / VPL;
   const int lanes = block / VPL;
   const unsigned grid = static_cast<unsigned>((words + kBlockThreads * kBlockUnroll - 1) / (kBlockThreads * kBlockUnroll));
 #define BQ_CASE(L)                                                                         \
   case L:                                                                                  \
-    hipLaunchKernelGGL((quantize_block_kernel<VPL, L, DYNAMIC>), dim3(grid), dim3(kBlockThreads), \
-                       0, st, x, words, out, scales_out, scales_in, sdt);                  \
+    hipLaunchKernelGGL((quantize_block_kernel<VPL, L, DYNAMIC, TWO>), dim3(grid), dim3(kBlockThreads), \
+                       0, st, x, words, out, scales_out, scales_in, sdt, stored_out);      \
     break;
   switch (lanes) {
     BQ_CASE(1) BQ_CASE(2) BQ_CASE(4) BQ_CASE(8) BQ_CASE(16) BQ_CASE(32) BQ_CASE(64)
@@ -668,6 +684,15 @@ two_level_split_kernel(float* __restrict__ scales, size_t n, const uint32_t* __r
   }
 }
 
+// The per-tensor scale from the absmax cells of the whole tensor. The largest block scale is the
+// scale of the largest block maximum (every step of scale = (2 absmax) / (b - a) is a correctly
+// rounded, hence monotonic, operation), so no block scale has to exist yet.
+__global__ void __launch_bounds__(kThreads)
+two_level_global_kernel(const uint32_t* __restrict__ cells, float span, float dtype_max, float* __restrict__ global_out) {
+  const float top = scale_from_absmax(absmax_from_cells(cells), span);
+  if (threadIdx.x == 0) global_out[0] = fmaxf(top / dtype_max, 1.17549435e-38f);
+}
+
 __global__ void scales_times_global_kernel(const float* __restrict__ stored, const float* __restrict__ global, size_t n,
                                            float* __restrict__ scales) {
   const size_t i = static_cast<size_t>(blockIdx.x) * blockDim.x + threadIdx.x;
@@ -684,6 +709,16 @@ bq_status launch_two_level_split(float* scales, size_t n, const uint32_t* cells,
   if (n == 0) return BQ_OK;
   hipLaunchKernelGGL(two_level_split_kernel, dim3(static_cast<unsigned>((n + kThreads - 1) / kThreads)), dim3(kThreads), 0, st,
                      scales, n, cells, sdt == BQ_SCALE_F16 ? 65504.0f : 448.0f, sdt, global_out, stored);
+  BQ_HIP(hipGetLastError());
+  return BQ_OK;
+}
+
+bq_status launch_two_level_global(const uint32_t* cells, int value, int sdt, float* global_out, hipStream_t st) {
+  if (sdt != BQ_SCALE_F16 && sdt != BQ_SCALE_UE4M3)
+    BQ_FAIL(BQ_ERR_UNSUPPORTED_SCHEME,
+            "block scales of this dtype reach f32's range, which a per-tensor scale cannot absorb (f16 and ue4m3 block scales can)");
+  hipLaunchKernelGGL(two_level_global_kernel, dim3(1), dim3(kThreads), 0, st, cells, 2.0f * static_cast<float>(value_qmax(value)),
+                     sdt == BQ_SCALE_F16 ? 65504.0f : 448.0f, global_out);
   BQ_HIP(hipGetLastError());
   return BQ_OK;
 }
@@ -970,6 +1005,16 @@ bq_status launch_quantize_run_block(const float* x, size_t n, int block, const f
                            : launch_block<8, true>(x, n, block, out, scales_out, nullptr, sdt, st);
   return value == BQ_Q8S ? launch_block<4, false>(x, n, block, out, nullptr, scales_in, sdt, st)
                          : launch_block<8, false>(x, n, block, out, nullptr, scales_in, sdt, st);
+}
+
+// quantize_dynamic of a two-level run-block scheme in one pass over x, given the per-tensor scale.
+bq_status launch_quantize_run_block_two_level(const float* x, size_t n, int block, const float* global, float* stored_out,
+                                              float* scales_out, int value, int store, void* values, int sdt, hipStream_t st) {
+  BQ_TRY(check_block_args(x, n, block, value, store, values));
+  if (n == 0) return BQ_OK;
+  uint32_t* out = static_cast<uint32_t*>(values);
+  return value == BQ_Q8S ? launch_block<4, true, true>(x, n, block, out, scales_out, global, sdt, st, stored_out)
+                         : launch_block<8, true, true>(x, n, block, out, scales_out, global, sdt, st, stored_out);
 }
 
 }  // namespace bq

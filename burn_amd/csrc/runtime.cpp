@@ -769,6 +769,24 @@ static bq_status quantize_impl(const bq_tensor* x, const bq_scheme* scheme, cons
   // over x (the values it writes are overwritten), splits them, and quantizes against the products.
   const int sdt = two_level ? BQ_SCALE_F32 : scheme->scale_dtype;
   bool dynamic_pass = dynamic;
+  // Run blocks with a fused kernel need no first pass: the largest block scale follows from the
+  // tensor's absmax alone, and the block kernel splits each scale as it computes it.
+  const long run = scheme->level == BQ_LEVEL_BLOCK ? run_block(*scheme, x->shape, x->rank) : 0;
+  if (two_level && dynamic && n > 0 && value_known(scheme->value) && run > 0 && run <= 512 &&
+      fused_block_ok(static_cast<int>(run), scheme->value)) {
+    uint32_t* cells = reinterpret_cast<uint32_t*>(q->scales() + q->num_scales);
+    rc = bqk_absmax_f32(xin, n, cells, st);
+    if (rc == BQ_OK) rc = launch_two_level_global(cells, scheme->value, scheme->scale_dtype, q->wire_global(), st);
+    if (rc == BQ_OK)
+      rc = launch_quantize_run_block_two_level(xin, n, static_cast<int>(run), q->wire_global(), q->wire_scales(), q->scales(),
+                                               scheme->value, scheme->store, q->data, scheme->scale_dtype, st);
+    if (rc != BQ_OK) {
+      bq_tensor_release(q);
+      return rc;
+    }
+    *out = q;
+    return BQ_OK;
+  }
   for (int pass = 0; pass < 2; ++pass) {
     if (pass == 1) {
       if (!(two_level && dynamic) || rc != BQ_OK || n == 0) break;

@@ -568,7 +568,10 @@ def test_layout_ops_known_answers(dev, approx):
                                          (QuantValue.Q4S, QuantStore.PackedU32)])
 @pytest.mark.parametrize("block", [None, (32,)])
 @pytest.mark.parametrize("shape,axes", [((24, 64), (1, 0)), ((3, 8, 64), (2, 0, 1)), ((2, 16, 3, 32), (0, 3, 2, 1)),
-                                        ((5, 32), (1, 0))])
+                                        ((5, 32), (1, 0)),
+                                        # the tiled transpose of 8-bit values: several tiles, ragged edges, batches
+                                        ((132, 288), (1, 0)), ((256, 128), (1, 0)), ((3, 2, 36, 160), (0, 1, 3, 2)),
+                                        ((4, 640), (1, 0)), ((2, 260, 32), (0, 2, 1))])
 def test_q_permute_matches_oracle(dev, value, store, block, shape, axes):
     """Values and block scales after q_permute are the oracle's, byte for byte on the wire, and
     dequantize commutes with the permutation bit for bit."""
@@ -999,6 +1002,13 @@ def test_q2s_ternary_matmul_is_the_reference_sum(dev):
         lin = FloatOps.float_into_data(ModuleOps.linear(FloatOps.float_from_data(x.reshape(1, m, k), dev), tw,
                                                         FloatOps.float_from_data(bias, dev)))
         assert lin.shape == (1, m, n) and lin.reshape(m, n).tobytes() == (got + bias).astype(np.float32).tobytes()
+    # infinite and NaN activations: a skipped field leaves the sum alone, +-1 adds or subtracts them
+    xs = rng.standard_normal((5, k)).astype(np.float32)
+    xs[0, 3], xs[1, 10], xs[2, 40], xs[3, 7], xs[3, 8] = np.inf, -np.inf, np.nan, np.inf, np.inf
+    got = FloatOps.float_into_data(QTensorOps.q_matmul(FloatOps.float_from_data(xs, dev), tw))
+    want = co.ternary_matmul(xs, q, s.reshape(-1)[0])
+    assert (np.isnan(got) == np.isnan(want)).all() and (got[~np.isnan(want)] == want[~np.isnan(want)]).all()
+    assert np.isinf(want).any() and np.isnan(want).any() and np.isfinite(want[4]).all()
     # per-block Q2S and bf16 activations take the dequantize route, like the reference
     twb = QTensorOps.quantize_dynamic(FloatOps.float_from_data(wr, dev), QuantScheme(value=QuantValue.Q2S).per_block((16,)))
     qb, sb = unpack_blob(QTensorOps.q_into_data(twb))
