@@ -143,6 +143,35 @@ def test_block_cache_rules(tmp_path):
     assert "block cache: ok" in out
 
 
+def c_driver():
+    """The plain-C caller of the ABI (tests/cpp/c_abi_driver.c), built by __graft_entry__.build()."""
+    exe = os.path.join(ROOT, "tests", "cpp", "c_abi_driver")
+    if not os.path.exists(exe):
+        import __graft_entry__
+        __graft_entry__.build_c_driver()
+    return exe
+
+
+def test_header_is_plain_c_and_a_c_caller_links():
+    """include/burnq.h compiles as C99 and as C++11, and a C program linked against the library
+    gets the reference's packed-Q4 blob lengths and the ABI's refusals without a GPU."""
+    import subprocess
+    hdr = os.path.join(ROOT, "include", "burnq.h")
+    subprocess.run(["gcc", "-std=c99", "-Wall", "-Wextra", "-pedantic", "-Werror", "-fsyntax-only", "-x", "c", hdr], check=True)
+    subprocess.run(["g++", "-std=c++11", "-Wall", "-Werror", "-fsyntax-only", "-x", "c++", hdr], check=True)
+    out = subprocess.run([c_driver(), "--no-gpu"], check=True, capture_output=True, text=True).stdout
+    assert "host-only cases ok" in out
+
+
+@pytest.mark.gpu
+def test_c_caller_runs_the_reference_cases_on_the_gpu():
+    """The same C program on the GPU: the reference's quantize / dequantize / pack / q_matmul
+    literals through the handle level of the ABI, no Python in between."""
+    import subprocess
+    r = subprocess.run([c_driver()], capture_output=True, text=True, timeout=120)
+    assert r.returncode == 0 and "all cases ok" in r.stdout, r.stdout + r.stderr
+
+
 def test_no_cpu_fallback():
     if ba.Device.count() > 0:
         pytest.skip("a GPU is present")
