@@ -37,6 +37,20 @@ static size_t num_elements(const size_t* shape, int rank) {
   return n;
 }
 
+// Shapes come from the caller: every size derived from one (element counts, byte counts, the
+// allocation) must fit comfortably in 64 bits before anything is multiplied. 2^44 elements is far
+// beyond the device's memory and leaves room for the factors applied later.
+static bq_status check_shape_size(const size_t* shape, int rank) {
+  const size_t limit = static_cast<size_t>(1) << 44;
+  size_t n = 1;
+  for (int d = 0; d < rank; ++d) {
+    if (shape[d] > limit || (shape[d] != 0 && n > limit / shape[d]))
+      BQ_FAIL(BQ_ERR_SIZE, "a shape of more than 2^44 elements (dim %d = %zu) is not addressable", d, shape[d]);
+    n *= shape[d];
+  }
+  return BQ_OK;
+}
+
 // params_shape (crates/burn-std/src/tensor/quantization.rs:141-146)
 static size_t num_params(const bq_scheme& s, const size_t* shape, int rank) {
   if (s.level == BQ_LEVEL_TENSOR) return 1;
@@ -70,6 +84,7 @@ static size_t global_size(const bq_scheme& s) { return s.tensor_scale ? 4 : 0; }
 // length formula alone (quantized_data_len) pads a ragged last dim to whole words instead.
 static bq_status check_scheme(const bq_scheme& s, const size_t* shape, int rank, bool storable = true) {
   if (rank < 1 || rank > BQ_MAX_RANK) BQ_FAIL(BQ_ERR_SHAPE, "rank %d outside 1..%d", rank, BQ_MAX_RANK);
+  BQ_TRY(check_shape_size(shape, rank));
   if (!value_supported(s.value))
     BQ_FAIL(BQ_ERR_UNSUPPORTED_SCHEME, "Quantization not supported for value %d (Q8S, Q4S and Q2S are)", s.value);
   if (s.scale_dtype > BQ_SCALE_UE4M3)
@@ -423,6 +438,7 @@ static bq_status new_float(bq_device* dev, int32_t dtype, const size_t* shape, i
                            bq_tensor** out) {
   if (dtype != BQ_F32 && dtype != BQ_BF16) BQ_FAIL(BQ_ERR_DTYPE, "float dtype must be f32 or bf16");
   if (rank < 1 || rank > BQ_MAX_RANK) BQ_FAIL(BQ_ERR_SHAPE, "rank %d outside 1..%d", rank, BQ_MAX_RANK);
+  BQ_TRY(check_shape_size(shape, rank));
   bq_tensor* t = new bq_tensor();
   t->dev = dev;
   t->dtype = dtype;
@@ -561,6 +577,7 @@ extern "C" bq_status bq_float_from_device_ptr(bq_device* dev, void* device_ptr, 
   BQ_NOTNULL(out);
   if (dtype != BQ_F32 && dtype != BQ_BF16) BQ_FAIL(BQ_ERR_DTYPE, "float dtype must be f32 or bf16");
   if (rank < 1 || rank > BQ_MAX_RANK) BQ_FAIL(BQ_ERR_SHAPE, "rank %d outside 1..%d", rank, BQ_MAX_RANK);
+  BQ_TRY(check_shape_size(shape, rank));
   bq_tensor* t = new bq_tensor();
   t->dev = dev;
   t->dtype = dtype;
@@ -1281,6 +1298,7 @@ extern "C" bq_status bq_q_reshape(const bq_tensor* t, const size_t* shape, int32
   BQ_NOTNULL(out);
   if (t->dtype != BQ_QFLOAT) BQ_FAIL(BQ_ERR_DTYPE, "q_reshape takes a quantized tensor");
   if (rank < 1 || rank > BQ_MAX_RANK) BQ_FAIL(BQ_ERR_SHAPE, "rank %d outside 1..%d", rank, BQ_MAX_RANK);
+  BQ_TRY(check_shape_size(shape, rank));
   if (num_elements(shape, rank) != t->numel())
     BQ_FAIL(BQ_ERR_SHAPE, "reshape changes the number of elements (%zu -> %zu)", t->numel(),
             num_elements(shape, rank));

@@ -116,6 +116,20 @@ def test_data_len_refuses_what_q_from_data_would_refuse():
     assert status(bad, (4, 64)) == _lib.ERR_UNSUPPORTED_SCHEME
 
 
+def test_shapes_whose_sizes_would_overflow_are_refused():
+    """Element and byte counts are products of caller-supplied dims: a shape past 2^44 elements is
+    refused before anything is multiplied (no wrapped-around allocation size)."""
+    L = _lib.lib()
+    n = C.c_size_t(0)
+    sch = QuantScheme().to_c()
+    for dims in ((1 << 33, 1 << 33), (1 << 62, 4), (3, 1 << 45)):
+        shape = (C.c_size_t * len(dims))(*dims)
+        assert L.bq_quantized_data_len(C.byref(sch), shape, len(dims), C.byref(n)) == _lib.ERR_SIZE
+        assert b"not addressable" in L.bq_last_error()
+    shape = (C.c_size_t * 2)(1 << 20, 1 << 20)   # 2^40 values: a length, not an allocation
+    assert L.bq_quantized_data_len(C.byref(sch), shape, 2, C.byref(n)) == _lib.OK and n.value == (1 << 40) + 4
+
+
 def test_static_scratch_entry_point_refuses_large_products_without_a_gpu():
     """bqk_q_linear_static checks the scratch it would need against the static array before
     anything else happens."""
