@@ -122,7 +122,7 @@ constexpr int kBlockUnroll = BQ_BLOCK_UNROLL;
 constexpr int kTensorUnroll = BQ_TENSOR_UNROLL;      // per-tensor second pass
 
 // Lane 4j + i of a workgroup of T threads holds words chunk + T u + 4j + i, u = 0..3. A 4 x 4
-// transpose inside each quad of lanes (two rounds of DPP swaps) leaves lane 4j + i with the four
+// transpose inside each quad of lanes (two DPP swaps) leaves lane 4j + i with the four
 // consecutive words chunk + T i + 4j + {0..3}: one 16-byte store per lane instead of four 4-byte
 // ones (1 % on the [8192, 8192] block quantize).
 template <int T>
@@ -131,12 +131,12 @@ __device__ __forceinline__ void store_words_quad(uint32_t (&packed)[4], size_t c
   auto swap1 = [](uint32_t v) { return static_cast<uint32_t>(__builtin_amdgcn_update_dpp(0, static_cast<int>(v), 0xB1, 0xF, 0xF, false)); };
   auto swap2 = [](uint32_t v) { return static_cast<uint32_t>(__builtin_amdgcn_update_dpp(0, static_cast<int>(v), 0x4E, 0xF, 0xF, false)); };
 #pragma unroll
-  for (int p = 0; p < 4; p += 2) {   // round 1: lanes i and i ^ 1 exchange across registers p, p + 1
+  for (int p = 0; p < 4; p += 2) {   // first: lanes i and i ^ 1 exchange across registers p, p + 1
     const uint32_t got = swap1(b0 ? packed[p] : packed[p + 1]);
     if (b0) packed[p] = got; else packed[p + 1] = got;
   }
 #pragma unroll
-  for (int p = 0; p < 2; ++p) {      // round 2: lanes i and i ^ 2 exchange across registers p, p + 2
+  for (int p = 0; p < 2; ++p) {      // then: lanes i and i ^ 2 exchange across registers p, p + 2
     const uint32_t got = swap2(b1 ? packed[p] : packed[p + 2]);
     if (b1) packed[p] = got; else packed[p + 2] = got;
   }

@@ -837,7 +837,11 @@ def test_two_level_quantize_dynamic(dev, sdt, value, store, shape, block, mag):
     x = (np.random.default_rng(len(shape) * 100 + shape[-1]).standard_normal(shape) * mag).astype(np.float32)
     scheme = QuantScheme(value=value, store=store).per_block(block, sdt).per_tensor(ScaleDtype.F32)
     assert scheme.tensor_scale == ScaleDtype.F32 and scheme.block == block
-    osch, code = oscheme(scheme), SDT[sdt][0]
+    check_two_level(dev, x, scheme)
+
+
+def check_two_level(dev, x, scheme):
+    osch, code = oscheme(scheme), SDT[scheme.scale_dtype][0]
     q_ref, stored_ref, g_ref, eff_ref = co.quantize_dynamic_two_level(x, osch, code)
     tq = QTensorOps.quantize_dynamic(FloatOps.float_from_data(x, dev), scheme)
     assert tq.scheme == scheme
@@ -845,12 +849,13 @@ def test_two_level_quantize_dynamic(dev, sdt, value, store, shape, block, mag):
     q, stored, g = two_level_parts(blob)
     assert g == g_ref and stored.tobytes() == stored_ref.tobytes() and (q == q_ref).all()
     assert blob.bytes.tobytes() == co.encode_two_level(q_ref, osch, stored_ref, g_ref, code).tobytes()
-    assert blob.bytes.size == TensorData.data_len(shape, scheme)
+    assert blob.bytes.size == TensorData.data_len(x.shape, scheme)
     d_ref = co.dequantize(q_ref, osch, eff_ref)
     assert FloatOps.float_into_data(QTensorOps.dequantize(tq)).tobytes() == d_ref.tobytes()
     again = QTensorOps.q_from_data(blob, dev)
     assert FloatOps.float_into_data(QTensorOps.dequantize(again)).tobytes() == d_ref.tobytes()
     assert QTensorOps.q_into_data(again).bytes.tobytes() == blob.bytes.tobytes()
+    return tq, q_ref, eff_ref
 
 
 def test_two_level_reference_cases(dev, approx):
@@ -893,6 +898,26 @@ def test_two_level_reference_cases(dev, approx):
     q_ref, stored_ref, g_ref, eff_ref = co.quantize_dynamic_two_level(big, oscheme(scheme), co.SCALE_F16)
     q, stored, g = two_level_parts(QTensorOps.q_into_data(tb))
     assert stored.max() == np.float32(65504.0) and g == g_ref and stored.tobytes() == stored_ref.tobytes() and (q == q_ref).all()
+
+
+def test_two_level_reference_scheme_cases(dev, approx):
+    """crates/burn-backend-tests/tests/tensor/float/quantization/scheme.rs:51-90 and 92-123, through
+    quantize_dynamic on inputs with those block ranges: the largest stored ue4m3 block scale is 448,
+    stored x global gives back the one-level scales (default tolerance); an all-zero tensor gets a
+    positive per-tensor scale and finite block scales."""
+    x = np.float32([-1.8, 0.5, 0, 0, -0.5, 1.8, 0, 0, 0.01, 0.04, 0.02, 0.03, -0.04, -0.01, -0.02, -0.03])
+    one = QuantScheme(store=QuantStore.Native).per_block((4,))
+    two = QuantScheme(store=QuantStore.Native).per_block((4,), ScaleDtype.UE4M3).per_tensor(ScaleDtype.F32)
+    expected = QTensorOps.q_into_data(QTensorOps.quantize_dynamic(FloatOps.float_from_data(x, dev), one)).split()[1]
+    approx(expected, np.float32([0.01417323, 0.01417323, 0.00031496, 0.00031496]))   # (scheme.rs:30-49)
+    blob = QTensorOps.q_into_data(QTensorOps.quantize_dynamic(FloatOps.float_from_data(x, dev), two))
+    _, stored, g = two_level_parts(blob)
+    approx(np.float32([stored.max()]), np.float32([448.0]))
+    approx(stored * g, expected)
+    z = QTensorOps.quantize_dynamic(FloatOps.float_from_data(np.zeros(4, np.float32), dev), two)
+    _, stored, g = two_level_parts(QTensorOps.q_into_data(z))
+    assert g > 0 and np.isfinite(stored).all()
+    assert (FloatOps.float_into_data(QTensorOps.dequantize(z)) == 0).all()
 
 
 def test_two_level_quantize_with_given_parameters_and_other_ops(dev, tmp_path):
@@ -1014,6 +1039,74 @@ def test_q2s_ternary_matmul_is_the_reference_sum(dev):
     qb, sb = unpack_blob(QTensorOps.q_into_data(twb))
     gotb = FloatOps.float_into_data(QTensorOps.q_matmul(FloatOps.float_from_data(x, dev), twb))
     matmul_check(gotb, no.q_matmul_f64(x, qb, sb, [16]))
+
+
+# ------------------------------------------------------------------ random schemes
+
+def random_scheme_case(rng):
+    """A quantizable (shape, scheme, magnitude): value, store, rank 1-4, per tensor or a block of rank
+    1-rank with power-of-two extents (whole packed words along the last dim), any scale dtype, the
+    two-level form for f16 / ue4m3 block scales."""
+    value = [QuantValue.Q8S, QuantValue.Q4S, QuantValue.Q2S][rng.integers(3)]
+    nq = {QuantValue.Q8S: 4, QuantValue.Q4S: 8, QuantValue.Q2S: 16}[value]
+    store = QuantStore.Native if value == QuantValue.Q8S and rng.integers(2) else QuantStore.PackedU32
+    rank = int(rng.integers(1, 5))
+    sdt = [ScaleDtype.F32, ScaleDtype.F16, ScaleDtype.BF16, ScaleDtype.UE4M3][rng.integers(4)]
+    block = None
+    if rng.integers(4):
+        br = int(rng.integers(1, rank + 1))
+        block = [int(2 ** rng.integers(0, 4)) for _ in range(br)]
+        block[-1] = int(nq * 2 ** rng.integers(0, 3)) if store == QuantStore.PackedU32 else int(2 ** rng.integers(0, 7))
+        block = tuple(block)
+    ext = [1] * rank
+    if block:
+        for j in range(len(block)):
+            ext[rank - 1 - j] = block[len(block) - 1 - j]
+    elif store == QuantStore.PackedU32:
+        ext[-1] = nq
+    shape = tuple(int(e * rng.integers(1, 4)) for e in ext)
+    scheme = QuantScheme(value=value, store=store, scale_dtype=sdt) if block is None else \
+        QuantScheme(value=value, store=store).per_block(block, sdt)
+    if block is not None and sdt in (ScaleDtype.F16, ScaleDtype.UE4M3) and rng.integers(2):
+        scheme = scheme.per_tensor(ScaleDtype.F32)
+    return shape, scheme, float(10.0 ** rng.integers(-4, 4))
+
+
+def test_random_schemes_against_the_oracle(dev):
+    """200 seeded cases over the whole scheme space: quantize_dynamic's blob, the dequantized floats
+    and the blob round trip bit for bit, then one layout op (swap / permute / flip) on the result,
+    whose dequantized values must be the same permutation of the source's."""
+    rng = np.random.default_rng(20240607)
+    seen = set()
+    for case in range(200):
+        shape, scheme, mag = random_scheme_case(rng)
+        x = (rng.standard_normal(shape) * mag).astype(np.float32)
+        if rng.integers(5) == 0:
+            x[rng.random(shape) < 0.3] = 0.0
+        label = f"case {case}: {shape} {scheme}"
+        try:
+            if scheme.tensor_scale is not None:
+                tq, _, _ = check_two_level(dev, x, scheme)
+            elif scheme.scale_dtype != ScaleDtype.F32:
+                tq, _, _ = check_scale_dtype(dev, x, scheme)
+            else:
+                tq, _, _, _ = check_quantize_dynamic(dev, x, scheme)
+        except AssertionError as e:
+            raise AssertionError(f"{label}: {e}") from e
+        seen.add((scheme.value, scheme.store, scheme.block is None, scheme.scale_dtype, scheme.tensor_scale))
+        d = FloatOps.float_into_data(QTensorOps.dequantize(tq))
+        rank = len(shape)
+        axes = [int(a) for a in rng.permutation(rank)]
+        nq = tq.scheme.num_quants()
+        if rank > 1 and (scheme.store == QuantStore.Native or scheme.value == QuantValue.Q8S or shape[axes[-1]] % nq == 0):
+            tp = QTensorOps.q_permute(tq, axes)
+            got = FloatOps.float_into_data(QTensorOps.dequantize(tp))
+            assert got.tobytes() == np.ascontiguousarray(np.transpose(d, axes)).tobytes(), f"{label}: permute {axes}"
+        fl = sorted({int(a) for a in rng.integers(0, rank, 2)})
+        if scheme.block is None:   # (a flip keeps block scales in place: only per-tensor values commute with it)
+            got = FloatOps.float_into_data(QTensorOps.dequantize(QTensorOps.q_flip(tq, fl)))
+            assert got.tobytes() == np.ascontiguousarray(np.flip(d, fl)).tobytes(), f"{label}: flip {fl}"
+    assert len(seen) >= 36   # of the 40 (value, store) x (level, scale dtype, two-level) combinations
 
 
 # ------------------------------------------------------------------ burnpack files
