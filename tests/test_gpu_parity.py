@@ -1109,6 +1109,76 @@ def test_random_schemes_against_the_oracle(dev):
     assert len(seen) >= 36   # of the 40 (value, store) x (level, scale dtype, two-level) combinations
 
 
+def test_random_matmuls_against_float64(dev):
+    """150 seeded products over the scheme space and the shapes that pick each kernel family: a float
+    (f32 / bf16) or quantized lhs, a quantized rhs of any scheme (any block shape, scale dtype,
+    two-level, ternary), batch dims that broadcast, M from 1 to 130. Against the float64 product of
+    the dequantized operands (dequantize itself is checked bit for bit elsewhere)."""
+    rng = np.random.default_rng(777)
+
+    def family_case():
+        """Weights shaped for the fused kernels: whole 128-column groups, K in 32-row steps (or not)."""
+        value = [QuantValue.Q8S, QuantValue.Q4S][rng.integers(2)]
+        store = QuantStore.Native if value == QuantValue.Q8S and rng.integers(3) == 0 else QuantStore.PackedU32
+        n = int([128, 256, 384, 640, 1024, 96, 48][rng.integers(7)])
+        k = int([32, 64, 96, 256, 512, 1000, 40][rng.integers(7)])
+        block = [None, (32,), (64,), (128,), (16,), (8,)][rng.integers(6)]
+        if block is not None and n % block[0]:
+            block = (16,)
+        sdt = [ScaleDtype.F32, ScaleDtype.F16, ScaleDtype.BF16, ScaleDtype.UE4M3][rng.integers(4)]
+        scheme = QuantScheme(value=value, store=store, scale_dtype=sdt) if block is None else \
+            QuantScheme(value=value, store=store).per_block(block, sdt)
+        if block is not None and sdt in (ScaleDtype.F16, ScaleDtype.UE4M3) and rng.integers(3) == 0:
+            scheme = scheme.per_tensor(ScaleDtype.F32)
+        batch = [(), (), (2,), (1, 3)][rng.integers(4)]
+        return batch + (k, n), scheme
+
+    for case in range(150):
+        shape, scheme, _ = random_scheme_case(rng)
+        if case % 2:
+            shape, scheme = family_case()
+        if len(shape) < 2:
+            shape = (int(rng.integers(1, 5)) * 8,) + shape
+            if scheme.block is not None and len(scheme.block) > 1:
+                scheme = QuantScheme(value=scheme.value, store=scheme.store).per_block(scheme.block[-1:], scheme.scale_dtype)
+        # a longer K now and then (the split-K and tiled kernels), keeping the block's divisibility
+        if case % 2 == 0 and rng.integers(3) == 0:
+            kb = 1
+            if scheme.block is not None and len(scheme.block) >= 2:
+                kb = scheme.block[-2]
+            shape = shape[:-2] + (shape[-2] * int(rng.integers(2, 9)) * (32 // np.gcd(32, kb) if rng.integers(2) else 1),) + shape[-1:]
+        rank = len(shape)
+        w = (rng.standard_normal(shape) * 0.02).astype(np.float32)
+        tw = QTensorOps.quantize_dynamic(FloatOps.float_from_data(w, dev), scheme)
+        wd = FloatOps.float_into_data(QTensorOps.dequantize(tw)).astype(np.float64)
+        m = int([1, 2, 3, 4, 5, 8, 16, 17, 32, 33, 64, 130][rng.integers(12)])
+        batch = tuple(1 if rng.integers(3) == 0 else b for b in shape[:-2])
+        xs = batch + (m, shape[-2])
+        xh = rng.standard_normal(xs).astype(np.float32)
+        kind = int(rng.integers(4))
+        label = f"case {case}: lhs {xs} kind {kind} x rhs {shape} {scheme}"
+        if kind == 0:      # f32 activations
+            lhs, xd = FloatOps.float_from_data(xh, dev), xh.astype(np.float64)
+        elif kind == 1:    # bf16 activations
+            bits = ba.bf16_bits_from_f32(xh)
+            lhs, xd = FloatOps.float_from_data(bits, dev, ba.BF16), ba.f32_from_bf16_bits(bits).astype(np.float64)
+        else:              # a quantized lhs (per tensor, or blocks along K)
+            k = xs[-1]
+            ls = QuantScheme(store=QuantStore.Native) if kind == 2 or k % 4 else QuantScheme().per_block((4,))
+            lhs = QTensorOps.quantize_dynamic(FloatOps.float_from_data(xh, dev), ls)
+            xd = FloatOps.float_into_data(QTensorOps.dequantize(lhs)).astype(np.float64)
+        ref = xd @ wd
+        try:
+            out = FloatOps.float_into_data(QTensorOps.q_matmul(lhs, tw, out_dtype=ba.F32))
+            assert out.shape == ref.shape
+            if np.abs(ref).max() == 0:
+                assert (out == 0).all()
+            else:
+                matmul_check(out, ref)
+        except (AssertionError, ba.BurnqError) as e:
+            raise AssertionError(f"{label}: {e}") from e
+
+
 # ------------------------------------------------------------------ burnpack files
 
 def test_burnpack_round_trip_of_device_tensors(dev, tmp_path):
