@@ -20,7 +20,7 @@ STATUS_NAMES = ["OK", "ERR_NULL", "ERR_UNSUPPORTED_SCHEME", "ERR_SHAPE", "ERR_DT
 # dtypes
 F32, BF16, QFLOAT = 0, 1, 2
 # scheme enums
-Q8S, Q4S, Q2S = 0, 1, 2
+Q8S, Q4S, Q2S, Q8F, Q4F, Q2F = 0, 1, 2, 3, 4, 5
 LEVEL_TENSOR, LEVEL_BLOCK = 0, 1
 STORE_NATIVE, STORE_PACKED_U32 = 0, 1
 SCALE_F32, SCALE_F16, SCALE_BF16, SCALE_UE4M3 = 0, 1, 2, 3

@@ -46,13 +46,20 @@ const char* get_error();
   } while (0)
 
 // ---- value helpers ---------------------------------------------------------------------------
-// QuantValue::range(): Q8S (-127,127), Q4S (-7,7), Q2S (-1,1) (ternary: -1, 0, +1).
-// value_known: what the fused kernels take. Q2S goes through the general kernels and the ternary
-// matmul only (value_supported).
-inline bool value_known(int v) { return v == BQ_Q8S || v == BQ_Q4S; }
-inline bool value_supported(int v) { return value_known(v) || v == BQ_Q2S; }
-inline int value_bits(int v) { return v == BQ_Q8S ? 8 : (v == BQ_Q4S ? 4 : 2); }
-inline int value_qmax(int v) { return v == BQ_Q8S ? 127 : (v == BQ_Q4S ? 7 : 1); }
+// QuantValue::range(): symmetric Q8S (-127,127), Q4S (-7,7), Q2S (-1,1) (ternary: -1, 0, +1);
+// full-range Q8F (-128,127), Q4F (-8,7), Q2F (-2,1). A full-range value has the bit layout of the
+// symmetric value of the same width (two's complement fields): only the quantize kernels -- the
+// span of the scale, the lower clamp -- tell them apart, everything else works on storage_value.
+inline bool value_supported(int v) { return v >= BQ_Q8S && v <= BQ_Q2F; }
+inline bool value_full(int v) { return v == BQ_Q8F || v == BQ_Q4F || v == BQ_Q2F; }
+inline int storage_value(int v) { return value_full(v) ? v - BQ_Q8F : v; }
+// value_known: what the fused kernels take (8- and 4-bit values). 2-bit values go through the
+// general kernels, Q2S also through the ternary matmul.
+inline bool value_known(int v) { return value_supported(v) && (storage_value(v) == BQ_Q8S || storage_value(v) == BQ_Q4S); }
+inline int value_bits(int v) { return storage_value(v) == BQ_Q8S ? 8 : (storage_value(v) == BQ_Q4S ? 4 : 2); }
+inline int value_qmax(int v) { return storage_value(v) == BQ_Q8S ? 127 : (storage_value(v) == BQ_Q4S ? 7 : 1); }  // b
+inline int value_qmin(int v) { return -value_qmax(v) - (value_full(v) ? 1 : 0); }                                   // a
+inline float value_span(int v) { return static_cast<float>(value_qmax(v) - value_qmin(v)); }                        // b - a
 inline int num_quants(int v) { return 32 / value_bits(v); }
 
 inline size_t round_up(size_t x, size_t a) { return (x + a - 1) / a * a; }

@@ -223,6 +223,7 @@ inline unsigned grid_for(size_t items, unsigned cap) {
 bq_status launch_dequantize_rect(const void* values, const size_t* shape, int rank,
                                  const size_t* blk, const float* scales, int value, int store,
                                  int out_dtype, void* out, hipStream_t st) {
+  value = storage_value(value);  // (a full-range value unpacks like its symmetric twin)
   RectDims d{};
   d.rank = blk ? rank : 0;
   size_t n = 1;
@@ -266,6 +267,7 @@ extern "C" bq_status bqk_dequantize(const void* values, size_t n, int32_t block,
   BQ_NOTNULL(scales);
   BQ_NOTNULL(out);
   if (!value_known(value)) BQ_FAIL(BQ_ERR_UNSUPPORTED_SCHEME, "unknown quant value %d", value);
+  value = storage_value(value);  // (a full-range value unpacks like its symmetric twin)
   if (out_dtype != BQ_F32 && out_dtype != BQ_BF16)
     BQ_FAIL(BQ_ERR_DTYPE, "dequantize target must be f32 or bf16");
   if (store == BQ_STORE_NATIVE && value != BQ_Q8S)

@@ -67,9 +67,9 @@ __device__ __forceinline__ int round_half_away_i32(float v) {
 }
 
 // Reference-order quantize of one value: IEEE divide, round half away, clamp.
-__device__ __forceinline__ int quantize_div(float x, float s, float qmax) {
+__device__ __forceinline__ int quantize_div(float x, float s, float qmin, float qmax) {
   float q = x / s;
-  q = fminf(fmaxf(q, -qmax), qmax);  // clamping before rounding is equivalent: bounds are integers
+  q = fminf(fmaxf(q, qmin), qmax);  // clamping before rounding is equivalent: bounds are integers
   return round_half_away_i32(q);
 }
 
@@ -115,9 +115,9 @@ __device__ __forceinline__ bool absmax_fast_ok(float amax) {
   return e >= 40u && e <= 220u;
 }
 
-__device__ __forceinline__ int quantize_recip(float x, float s, float r, float qmax) {
+__device__ __forceinline__ int quantize_recip(float x, float s, float r, float qmin, float qmax) {
   float q = div_by_recip(x, s, r);
-  q = fminf(fmaxf(q, -qmax), qmax);
+  q = fminf(fmaxf(q, qmin), qmax);
   return round_half_away_i32(q);
 }
 

@@ -138,6 +138,7 @@ GatherDims make_dims(const size_t* src_shape, int rank, const int32_t* axes, con
 // Values are i8 (native) or packed u32 words along the last dim; shapes are element shapes.
 bq_status launch_q_gather(const void* src, void* dst, const size_t* src_shape, int rank, const int32_t* axes,
                           const uint8_t* flip, int value, bool native, hipStream_t st) {
+  value = storage_value(value);  // (only the width of a field matters here)
   size_t n = 1;
   for (int a = 0; a < rank; ++a) n *= src_shape[a];
   if (n == 0) return BQ_OK;

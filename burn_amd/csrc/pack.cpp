@@ -166,7 +166,8 @@ int dtype_from_name(const std::string& s) {
 
 void write_scheme(CborWriter& w, const bq_scheme& s) {
   w.map(s.tensor_scale ? 6 : 5);
-  w.text("value"); w.text(s.value == BQ_Q8S ? "Q8S" : s.value == BQ_Q4S ? "Q4S" : "Q2S");
+  static const char* const kValueNames[] = {"Q8S", "Q4S", "Q2S", "Q8F", "Q4F", "Q2F"};
+  w.text("value"); w.text(kValueNames[s.value <= BQ_Q2F ? s.value : 0]);
   w.text("level");
   if (s.level == BQ_LEVEL_TENSOR) { w.text("Tensor"); }
   else { w.map(1); w.text("Block"); w.array(s.block_rank); for (int i = 0; i < s.block_rank; ++i) w.uint(s.block[i]); }
@@ -184,7 +185,8 @@ bool read_scheme(const Cbor& c, bq_scheme* s) {
   const Cbor *value = c.get("value"), *level = c.get("level"), *store = c.get("store"), *sd = c.get("scale_dtype");
   if (!value || !level || !store || !sd || value->kind != Cbor::Text || sd->kind != Cbor::Text) return false;
   if (value->s == "Q8S") s->value = BQ_Q8S; else if (value->s == "Q4S") s->value = BQ_Q4S;
-  else if (value->s == "Q2S") s->value = BQ_Q2S; else return false;
+  else if (value->s == "Q2S") s->value = BQ_Q2S; else if (value->s == "Q8F") s->value = BQ_Q8F;
+  else if (value->s == "Q4F") s->value = BQ_Q4F; else if (value->s == "Q2F") s->value = BQ_Q2F; else return false;
   if (const Cbor* ts = c.get("tensor_scale")) {
     if (ts->kind != Cbor::Text || ts->s != "F32") return false;
     s->tensor_scale = 1;

@@ -647,6 +647,7 @@ static size_t split_from_m(int value) { return value == BQ_Q8S ? 4 : 3; }
 namespace bq {
 // Whether bqk_q_matmul has a fused kernel for this problem (else: dequantize + float matmul).
 bool fused_matmul_ok(size_t m, size_t k, size_t n, int lhs_dtype, int value, size_t scales_per_row) {
+  value = storage_value(value);
   // (one or two rows of bf16 activations: the decode kernel, whatever K's divisibility by 8)
   const int block = scales_per_row ? static_cast<int>(n / scales_per_row) : 0;
   const bool bf16_decode = lhs_dtype == BQ_BF16 && k % 2 == 0 && gemv1_ok(m, n, lhs_dtype, block, value);
@@ -658,6 +659,7 @@ bool fused_matmul_ok(size_t m, size_t k, size_t n, int lhs_dtype, int value, siz
 extern "C" size_t bqk_q_matmul_workspace(size_t m, size_t k, size_t n, int32_t lhs_dtype,
                                          int32_t value) {
   if (!value_known(value) || m == 0 || n == 0 || k == 0) return 0;
+  value = storage_value(value);  // (the products read two's complement fields: full-range values are their symmetric twins here)
   // the block size and the alignment (which pick the kernel) are not known here: cover every plan
   size_t bytes = 0;
   if (skinny_ok(m, k, n, lhs_dtype, value)) bytes = skinny_workspace(m, k, n, lhs_dtype, value);
@@ -711,6 +713,7 @@ static bq_status q_matmul_core(const void* lhs, int32_t lhs_dtype, size_t m, siz
   BQ_NOTNULL(w_scales);
   BQ_NOTNULL(out);
   if (!value_known(value)) BQ_FAIL(BQ_ERR_UNSUPPORTED_SCHEME, "unknown quant value %d", value);
+  value = storage_value(value);  // (the products read two's complement fields: full-range values are their symmetric twins here)
   if (lhs_dtype != BQ_F32 && lhs_dtype != BQ_BF16) BQ_FAIL(BQ_ERR_DTYPE, "lhs must be f32 or bf16");
   if (out_dtype != BQ_F32 && out_dtype != BQ_BF16) BQ_FAIL(BQ_ERR_DTYPE, "out must be f32 or bf16");
   if (store == BQ_STORE_NATIVE && value != BQ_Q8S)

@@ -73,37 +73,39 @@ __device__ __forceinline__ float absmax_vals(const Vals<VPL>& a) {
 
 // Reference-order path: an IEEE divide per value. Taken for scales outside the exponent range
 // the reciprocal path is proven for (subnormal / huge scales) -- rare, so speed is irrelevant.
-template <int VPL>
+// FULL: a full-range value (Q8F, Q4F): the lower clamp is -QMAX - 1.
+template <int VPL, bool FULL = false>
 __device__ __forceinline__ uint32_t quantize_pack_div(const Vals<VPL>& a, float s) {
-  constexpr float QMAX = (VPL == 4) ? 127.0f : 7.0f;
+  constexpr float QMAX = (VPL == 4) ? 127.0f : 7.0f, QMIN = FULL ? -QMAX - 1.0f : -QMAX;
   int q[VPL];
 #pragma unroll
-  for (int i = 0; i < VPL; ++i) q[i] = quantize_div(a.v[i], s, QMAX);
+  for (int i = 0; i < VPL; ++i) q[i] = quantize_div(a.v[i], s, QMIN, QMAX);
   return pack_fields<VPL>(q);
 }
 
 // Fast path: quotients through r = RN(1/s) and one fma correction (== the IEEE quotient).
 // CLAMP is dropped when s came from this block's own absmax: |x| <= amax and
 // s = RN(amax / QMAX) is normal, so |x / s| < QMAX + 0.5 already.
-template <int VPL, bool CLAMP>
+// (A full-range value always clamps: absmax / s is QMAX + 0.5, which rounds to QMAX + 1.)
+template <int VPL, bool CLAMP, bool FULL = false>
 __device__ __forceinline__ uint32_t quantize_pack_recip(const Vals<VPL>& a, float s, float r) {
-  constexpr float QMAX = (VPL == 4) ? 127.0f : 7.0f;
+  constexpr float QMAX = (VPL == 4) ? 127.0f : 7.0f, QMIN = FULL ? -QMAX - 1.0f : -QMAX;
   int q[VPL];
 #pragma unroll
   for (int i = 0; i < VPL; ++i) {
     float v = div_by_recip(a.v[i], s, r);
-    if (CLAMP) v = fminf(fmaxf(v, -QMAX), QMAX);
+    if (CLAMP || FULL) v = fminf(fmaxf(v, QMIN), QMAX);
     q[i] = round_half_away_i32(v);
   }
   return pack_fields<VPL>(q);
 }
 
 // Quantize VPL values against a given (stored) scale.
-template <int VPL>
+template <int VPL, bool FULL = false>
 __device__ __forceinline__ uint32_t quantize_pack(const Vals<VPL>& a, float s_stored) {
   const float s = valid_scale(s_stored);
-  if (recip_path_ok(s)) return quantize_pack_recip<VPL, true>(a, s, recip_exact(s));
-  return quantize_pack_div<VPL>(a, s);
+  if (recip_path_ok(s)) return quantize_pack_recip<VPL, true, FULL>(a, s, recip_exact(s));
+  return quantize_pack_div<VPL, FULL>(a, s);
 }
 
 // ---- run-block schemes: B = LANES * VPL consecutive elements per scale ------------------------
@@ -151,7 +153,9 @@ __device__ __forceinline__ void store_words_quad(uint32_t (&packed)[4], size_t c
 // in the dtype `sdt`, and the block is quantized against global * that, which goes to `scales_out`
 // -- normalize_scales (crates/burn-backend/src/quantization/scheme.rs:106-134) and what
 // NdArray::quantize makes of its result, one IEEE operation per step as there.
-template <int VPL, int LANES, bool DYNAMIC, bool TWO = false>
+// FULL: a full-range value: span b - a = 2 QMAX + 1 (no proven divide-free form: the scale takes
+// the IEEE division, once per block), lower clamp -QMAX - 1.
+template <int VPL, int LANES, bool DYNAMIC, bool TWO = false, bool FULL = false>
 __global__ void __launch_bounds__(kBlockThreads)
 quantize_block_kernel(const float* __restrict__ x, size_t words, uint32_t* __restrict__ out,
                       float* __restrict__ scales_out, const float* __restrict__ scales_in, int sdt,
@@ -159,7 +163,7 @@ quantize_block_kernel(const float* __restrict__ x, size_t words, uint32_t* __res
   static_assert(!TWO || DYNAMIC, "two-level scales are split where the block scales are computed");
   constexpr int U = kBlockUnroll;
   constexpr int QMAX = (VPL == 4) ? 127 : 7;
-  constexpr float SPAN = 2.0f * QMAX;
+  constexpr float SPAN = 2.0f * QMAX + (FULL ? 1.0f : 0.0f);
   const size_t base = static_cast<size_t>(blockIdx.x) * (kBlockThreads * U) + threadIdx.x;
   constexpr bool kQuadStore = BQ_QUANT_QUAD_STORE && U == 4;
   uint32_t packed[U];
@@ -184,14 +188,17 @@ quantize_block_kernel(const float* __restrict__ x, size_t words, uint32_t* __res
     float stored = 0.0f;
     if (TWO) {
       const float m = group_max<LANES>(absmax_vals<VPL>(a[u]));
-      const float one_level = absmax_fast_ok(m) ? scale_from_absmax_fast<QMAX>(m) : scale_from_absmax(m, SPAN);
+      const float one_level = (!FULL && absmax_fast_ok(m)) ? scale_from_absmax_fast<QMAX>(m) : scale_from_absmax(m, SPAN);
       const float global = scales_in[0];
       stored = scale_round_up(one_level / global, sdt);
       s = global * stored;
-      word = quantize_pack<VPL>(a[u], s);
+      word = quantize_pack<VPL, FULL>(a[u], s);
     } else if (DYNAMIC) {
       const float m = group_max<LANES>(absmax_vals<VPL>(a[u]));
-      if (sdt != BQ_SCALE_F32) {  // f16 / bf16 scales: divide by the scale as it will be stored
+      if (FULL) {
+        s = scale_round_up(scale_from_absmax(m, SPAN), sdt);
+        word = quantize_pack<VPL, true>(a[u], s);
+      } else if (sdt != BQ_SCALE_F32) {  // f16 / bf16 scales: divide by the scale as it will be stored
         s = scale_round_up(absmax_fast_ok(m) ? scale_from_absmax_fast<QMAX>(m) : scale_from_absmax(m, SPAN), sdt);
         word = quantize_pack<VPL>(a[u], s);
       } else if (absmax_fast_ok(m)) {
@@ -203,7 +210,7 @@ quantize_block_kernel(const float* __restrict__ x, size_t words, uint32_t* __res
       }
     } else {
       s = (w < words) ? scales_in[w / LANES] : 1.0f;
-      word = quantize_pack<VPL>(a[u], s);
+      word = quantize_pack<VPL, FULL>(a[u], s);
     }
     if (w < words) {
       if (DYNAMIC && (w & (LANES - 1)) == 0) scales_out[w / LANES] = s;
@@ -315,13 +322,13 @@ __global__ void scales_from_absmax_kernel(const float* __restrict__ amax, size_t
 // FROM_ABSMAX: `scale` points at the absmax cells (bit patterns of partial max|x|) instead of a
 // scale; the scale is derived here, (2 * amax) / (b - a), and block 0 stores it to scale_out.
 // Same chunked layout as the block kernel.
-template <int VPL, bool FROM_ABSMAX>
+template <int VPL, bool FROM_ABSMAX, bool FULL = false>
 __global__ void __launch_bounds__(kThreads)
 quantize_tensor_kernel(const float* __restrict__ x, size_t n, const float* __restrict__ scale,
                        float* __restrict__ scale_out, uint32_t* __restrict__ out, int sdt) {
   constexpr int U = kTensorUnroll;
-  constexpr float SPAN = (VPL == 4) ? 254.0f : 14.0f;
-  constexpr float QMAX = (VPL == 4) ? 127.0f : 7.0f;
+  constexpr float QMAX = (VPL == 4) ? 127.0f : 7.0f, QMIN = FULL ? -QMAX - 1.0f : -QMAX;
+  constexpr float SPAN = QMAX - QMIN;
   const size_t words = n / VPL;
   const size_t base = static_cast<size_t>(blockIdx.x) * (kThreads * U) + threadIdx.x;
   Vals<VPL> a[U];
@@ -353,7 +360,7 @@ quantize_tensor_kernel(const float* __restrict__ x, size_t n, const float* __res
     packed[u] = 0u;
     if (w < words)
     {
-      packed[u] = fast ? quantize_pack_recip<VPL, true>(a[u], s, r) : quantize_pack_div<VPL>(a[u], s);
+      packed[u] = fast ? quantize_pack_recip<VPL, true, FULL>(a[u], s, r) : quantize_pack_div<VPL, FULL>(a[u], s);
       if (!quad) {
         if (BQ_QUANT_NT_STORE) __builtin_nontemporal_store(packed[u], out + w); else out[w] = packed[u];
       }
@@ -363,18 +370,18 @@ quantize_tensor_kernel(const float* __restrict__ x, size_t n, const float* __res
   // native i8 store with n % 4 != 0: the last 1..3 values, one byte each
   if (VPL == 4 && blockIdx.x == 0 && threadIdx.x == 0) {
     int8_t* bytes = reinterpret_cast<int8_t*>(out);
-    for (size_t i = words * 4; i < n; ++i) bytes[i] = static_cast<int8_t>(quantize_div(x[i], s, QMAX));
+    for (size_t i = words * 4; i < n; ++i) bytes[i] = static_cast<int8_t>(quantize_div(x[i], s, QMIN, QMAX));
   }
 }
 
 // Unaligned input pointer: one value per lane, byte stores (native Q8S only).
 __global__ void __launch_bounds__(kThreads)
 quantize_tensor_scalar_kernel(const float* __restrict__ x, size_t n,
-                              const float* __restrict__ scale, int8_t* __restrict__ out) {
+                              const float* __restrict__ scale, float qmin, int8_t* __restrict__ out) {
   const float s = valid_scale(scale[0]);
   const size_t stride = static_cast<size_t>(gridDim.x) * kThreads;
   for (size_t i = static_cast<size_t>(blockIdx.x) * kThreads + threadIdx.x; i < n; i += stride)
-    out[i] = static_cast<int8_t>(quantize_div(x[i], s, 127.0f));
+    out[i] = static_cast<int8_t>(quantize_div(x[i], s, qmin, 127.0f));
 }
 
 // ---- general rectangle blocks (any block shape): complete, not fast ---------------------------
@@ -426,10 +433,11 @@ __global__ void rect_scales_kernel(const float* __restrict__ x, RectDims d, size
 // One thread per output word; every value looks its own block up, so words may straddle blocks.
 template <int BITS>
 __global__ void rect_quantize_kernel(const float* __restrict__ x, RectDims d, size_t last,
-                                     size_t words_per_line, size_t total_words, bool native,
+                                     size_t words_per_line, size_t total_words, bool native, bool full,
                                      const float* __restrict__ scales, uint32_t* __restrict__ out) {
   constexpr int NQ = 32 / BITS;
   constexpr float QMAX = (BITS == 8) ? 127.0f : (BITS == 4 ? 7.0f : 1.0f);
+  const float QMIN = full ? -QMAX - 1.0f : -QMAX;
   constexpr uint32_t MASK = (1u << BITS) - 1u;
   size_t w = static_cast<size_t>(blockIdx.x) * blockDim.x + threadIdx.x;
   if (w >= total_words) return;
@@ -440,7 +448,7 @@ __global__ void rect_quantize_kernel(const float* __restrict__ x, RectDims d, si
     if (c >= last) break;
     size_t idx = line * last + c;
     float s = valid_scale(scales[d.rank ? rect_block_of(d, idx) : 0]);
-    int q = quantize_div(x[idx], s, QMAX);
+    int q = quantize_div(x[idx], s, QMIN, QMAX);
     if (native) {
       reinterpret_cast<int8_t*>(out)[idx] = static_cast<int8_t>(q);
     } else {
@@ -456,7 +464,7 @@ inline unsigned grid_for(size_t items, unsigned cap) {
   return static_cast<unsigned>(g < cap ? g : cap);
 }
 
-template <int VPL, bool DYNAMIC, bool TWO = false>
+template <int VPL, bool DYNAMIC, bool TWO = false, bool FULL = false>
 bq_status launch_block(const float* x, size_t n, int block, uint32_t* out, float* scales_out,
                        const float* scales_in, int sdt, hipStream_t st, float* stored_out = nullptr) {
   const size_t words = n / VPL;
@@ -464,7 +472,7 @@ bq_status launch_block(const float* x, size_t n, int block, uint32_t* out, float
   const unsigned grid = static_cast<unsigned>((words + kBlockThreads * kBlockUnroll - 1) / (kBlockThreads * kBlockUnroll));
 #define BQ_CASE(L)                                                                         \
   case L:                                                                                  \
-    hipLaunchKernelGGL((quantize_block_kernel<VPL, L, DYNAMIC, TWO>), dim3(grid), dim3(kBlockThreads), \
+    hipLaunchKernelGGL((quantize_block_kernel<VPL, L, DYNAMIC, TWO, FULL>), dim3(grid), dim3(kBlockThreads), \
                        0, st, x, words, out, scales_out, scales_in, sdt, stored_out);      \
     break;
   switch (lanes) {
@@ -560,7 +568,7 @@ bq_status launch_quantize_rect(const float* x, const size_t* shape, int rank, co
     block_elems *= d.blk[i];
   }
   if (n == 0) return BQ_OK;
-  const float span = 2.0f * static_cast<float>(value_qmax(value));
+  const float span = value_span(value);
   if (dynamic) {
     RectDims dd = d;
     dd.rank = rank;  // per-tensor: one block spanning everything
@@ -574,14 +582,15 @@ bq_status launch_quantize_rect(const float* x, const size_t* shape, int rank, co
   const size_t total = (n / last) * wpl;
   const bool native = store == BQ_STORE_NATIVE;
   dim3 grid((total + kThreads - 1) / kThreads), tb(kThreads);
-  if (value == BQ_Q8S)
-    hipLaunchKernelGGL(rect_quantize_kernel<8>, grid, tb, 0, st, x, d, last, wpl, total, native,
+  const bool full = value_full(value);
+  if (value_bits(value) == 8)
+    hipLaunchKernelGGL(rect_quantize_kernel<8>, grid, tb, 0, st, x, d, last, wpl, total, native, full,
                        scales, static_cast<uint32_t*>(values));
-  else if (value == BQ_Q4S)
-    hipLaunchKernelGGL(rect_quantize_kernel<4>, grid, tb, 0, st, x, d, last, wpl, total, native,
+  else if (value_bits(value) == 4)
+    hipLaunchKernelGGL(rect_quantize_kernel<4>, grid, tb, 0, st, x, d, last, wpl, total, native, full,
                        scales, static_cast<uint32_t*>(values));
   else
-    hipLaunchKernelGGL(rect_quantize_kernel<2>, grid, tb, 0, st, x, d, last, wpl, total, native,
+    hipLaunchKernelGGL(rect_quantize_kernel<2>, grid, tb, 0, st, x, d, last, wpl, total, native, full,
                        scales, static_cast<uint32_t*>(values));
   BQ_HIP(hipGetLastError());
   return BQ_OK;
@@ -656,7 +665,7 @@ __global__ void scales_from_wire_kernel(const T* __restrict__ src, float* __rest
 }
 
 bq_status launch_scale_from_cells(const uint32_t* cells, int value, int sdt, float* scale_out, hipStream_t st) {
-  hipLaunchKernelGGL(scale_from_cells_kernel, dim3(1), dim3(kThreads), 0, st, cells, 2.0f * static_cast<float>(value_qmax(value)),
+  hipLaunchKernelGGL(scale_from_cells_kernel, dim3(1), dim3(kThreads), 0, st, cells, value_span(value),
                      sdt, scale_out);
   BQ_HIP(hipGetLastError());
   return BQ_OK;
@@ -717,7 +726,7 @@ bq_status launch_two_level_global(const uint32_t* cells, int value, int sdt, flo
   if (sdt != BQ_SCALE_F16 && sdt != BQ_SCALE_UE4M3)
     BQ_FAIL(BQ_ERR_UNSUPPORTED_SCHEME,
             "block scales of this dtype reach f32's range, which a per-tensor scale cannot absorb (f16 and ue4m3 block scales can)");
-  hipLaunchKernelGGL(two_level_global_kernel, dim3(1), dim3(kThreads), 0, st, cells, 2.0f * static_cast<float>(value_qmax(value)),
+  hipLaunchKernelGGL(two_level_global_kernel, dim3(1), dim3(kThreads), 0, st, cells, value_span(value),
                      sdt == BQ_SCALE_F16 ? 65504.0f : 448.0f, global_out);
   BQ_HIP(hipGetLastError());
   return BQ_OK;
@@ -805,7 +814,7 @@ __global__ void selftest_quotient_kernel(unsigned long long* __restrict__ mismat
         const float x = __uint_as_float(tb + static_cast<uint32_t>(d));  // neighbours in magnitude
         const float exact = x / s, fast = div_by_recip(x, s, r);
         bad_q += __float_as_uint(exact) != __float_as_uint(fast);
-        bad_i += quantize_div(x, s, 127.0f) != quantize_recip(x, s, r, 127.0f);
+        bad_i += quantize_div(x, s, -127.0f, 127.0f) != quantize_recip(x, s, r, -127.0f, 127.0f);
       }
     }
   }
@@ -845,7 +854,7 @@ extern "C" bq_status bqk_scales_from_absmax(const float* absmax, size_t n, int32
   BQ_NOTNULL(scales);
   if (!value_known(value)) BQ_FAIL(BQ_ERR_UNSUPPORTED_SCHEME, "unknown quant value %d", value);
   if (n == 0) return BQ_OK;
-  const float span = 2.0f * static_cast<float>(value_qmax(value));
+  const float span = value_span(value);
   hipLaunchKernelGGL(scales_from_absmax_kernel, dim3((n + 255) / 256), dim3(256), 0,
                      static_cast<hipStream_t>(stream), absmax, n, span, scales);
   BQ_HIP(hipGetLastError());
@@ -855,7 +864,7 @@ extern "C" bq_status bqk_scales_from_absmax(const float* absmax, size_t n, int32
 static bq_status check_value_store(int32_t value, int32_t store, size_t n) {
   if (!value_known(value)) BQ_FAIL(BQ_ERR_UNSUPPORTED_SCHEME, "unknown quant value %d", value);
   if (store == BQ_STORE_NATIVE) {
-    if (value != BQ_Q8S)
+    if (value_bits(value) != 8)
       BQ_FAIL(BQ_ERR_UNSUPPORTED_SCHEME, "Can't store native sub-byte values");
   } else if (store == BQ_STORE_PACKED_U32) {
     if (n % static_cast<size_t>(num_quants(value)))
@@ -873,16 +882,17 @@ static bq_status quantize_per_tensor_impl(const float* x, size_t n, const float*
                                           int32_t store, void* values, int sdt, hipStream_t st) {
   BQ_TRY(check_value_store(value, store, n));
   if (n == 0) return BQ_OK;
+  const bool full = value_full(value), eight = value_bits(value) == 8;
   if (!aligned16(x) || (reinterpret_cast<uintptr_t>(values) & 3u)) {
-    if (value != BQ_Q8S)
-      BQ_FAIL(BQ_ERR_SHAPE, "Q4S quantize needs a 16-byte aligned input and 4-byte aligned output");
+    if (!eight)
+      BQ_FAIL(BQ_ERR_SHAPE, "4-bit quantize needs a 16-byte aligned input and 4-byte aligned output");
     if (from_absmax) {
       hipLaunchKernelGGL(scale_from_cells_kernel, dim3(1), dim3(kThreads), 0, st,
-                         reinterpret_cast<const uint32_t*>(scale), 254.0f, sdt, scale_out);
+                         reinterpret_cast<const uint32_t*>(scale), value_span(value), sdt, scale_out);
       scale = scale_out;
     }
     hipLaunchKernelGGL(quantize_tensor_scalar_kernel, dim3(grid_for(n, 65536u)), dim3(kThreads), 0, st, x,
-                       n, scale, static_cast<int8_t*>(values));
+                       n, scale, static_cast<float>(value_qmin(value)), static_cast<int8_t*>(values));
     BQ_HIP(hipGetLastError());
     return BQ_OK;
   }
@@ -892,17 +902,15 @@ static bq_status quantize_per_tensor_impl(const float* x, size_t n, const float*
   if (g < 1) g = 1;
   dim3 grid(static_cast<unsigned>(g)), tb(kThreads);
   uint32_t* out = static_cast<uint32_t*>(values);
-  if (value == BQ_Q8S) {
-    if (from_absmax)
-      hipLaunchKernelGGL((quantize_tensor_kernel<4, true>), grid, tb, 0, st, x, n, scale, scale_out, out, sdt);
-    else
-      hipLaunchKernelGGL((quantize_tensor_kernel<4, false>), grid, tb, 0, st, x, n, scale, scale_out, out, sdt);
+#define BQ_TENSOR(V, A, F) hipLaunchKernelGGL((quantize_tensor_kernel<V, A, F>), grid, tb, 0, st, x, n, scale, scale_out, out, sdt)
+  if (eight) {
+    if (from_absmax) { if (full) BQ_TENSOR(4, true, true); else BQ_TENSOR(4, true, false); }
+    else { if (full) BQ_TENSOR(4, false, true); else BQ_TENSOR(4, false, false); }
   } else {
-    if (from_absmax)
-      hipLaunchKernelGGL((quantize_tensor_kernel<8, true>), grid, tb, 0, st, x, n, scale, scale_out, out, sdt);
-    else
-      hipLaunchKernelGGL((quantize_tensor_kernel<8, false>), grid, tb, 0, st, x, n, scale, scale_out, out, sdt);
+    if (from_absmax) { if (full) BQ_TENSOR(8, true, true); else BQ_TENSOR(8, true, false); }
+    else { if (full) BQ_TENSOR(8, false, true); else BQ_TENSOR(8, false, false); }
   }
+#undef BQ_TENSOR
   BQ_HIP(hipGetLastError());
   return BQ_OK;
 }
@@ -943,6 +951,18 @@ static bq_status check_block_args(const float* x, size_t n, int32_t block, int32
   return BQ_OK;
 }
 
+// The run-block kernel for a value: 8- or 4-bit fields, symmetric or full range.
+template <bool DYNAMIC, bool TWO = false>
+static bq_status launch_block_for(int value, const float* x, size_t n, int block, uint32_t* out, float* scales_out,
+                                  const float* scales_in, int sdt, hipStream_t st, float* stored_out = nullptr) {
+  const bool full = value_full(value);
+  if (value_bits(value) == 8)
+    return full ? launch_block<4, DYNAMIC, TWO, true>(x, n, block, out, scales_out, scales_in, sdt, st, stored_out)
+                : launch_block<4, DYNAMIC, TWO, false>(x, n, block, out, scales_out, scales_in, sdt, st, stored_out);
+  return full ? launch_block<8, DYNAMIC, TWO, true>(x, n, block, out, scales_out, scales_in, sdt, st, stored_out)
+              : launch_block<8, DYNAMIC, TWO, false>(x, n, block, out, scales_out, scales_in, sdt, st, stored_out);
+}
+
 extern "C" bq_status bqk_quantize_dynamic_block(const float* x, size_t n, int32_t block,
                                                 int32_t value, int32_t store, void* values,
                                                 float* scales, void* stream) {
@@ -951,10 +971,8 @@ extern "C" bq_status bqk_quantize_dynamic_block(const float* x, size_t n, int32_
   BQ_NOTNULL(scales);
   BQ_TRY(check_block_args(x, n, block, value, store, values));
   if (n == 0) return BQ_OK;
-  hipStream_t st = static_cast<hipStream_t>(stream);
-  if (value == BQ_Q8S)
-    return launch_block<4, true>(x, n, block, static_cast<uint32_t*>(values), scales, nullptr, BQ_SCALE_F32, st);
-  return launch_block<8, true>(x, n, block, static_cast<uint32_t*>(values), scales, nullptr, BQ_SCALE_F32, st);
+  return launch_block_for<true>(value, x, n, block, static_cast<uint32_t*>(values), scales, nullptr, BQ_SCALE_F32,
+                                static_cast<hipStream_t>(stream));
 }
 
 extern "C" bq_status bqk_quantize_block(const float* x, size_t n, int32_t block,
@@ -965,10 +983,8 @@ extern "C" bq_status bqk_quantize_block(const float* x, size_t n, int32_t block,
   BQ_NOTNULL(scales);
   BQ_TRY(check_block_args(x, n, block, value, store, values));
   if (n == 0) return BQ_OK;
-  hipStream_t st = static_cast<hipStream_t>(stream);
-  if (value == BQ_Q8S)
-    return launch_block<4, false>(x, n, block, static_cast<uint32_t*>(values), nullptr, scales, BQ_SCALE_F32, st);
-  return launch_block<8, false>(x, n, block, static_cast<uint32_t*>(values), nullptr, scales, BQ_SCALE_F32, st);
+  return launch_block_for<false>(value, x, n, block, static_cast<uint32_t*>(values), nullptr, scales, BQ_SCALE_F32,
+                                 static_cast<hipStream_t>(stream));
 }
 
 
@@ -1000,11 +1016,8 @@ bq_status launch_quantize_run_block(const float* x, size_t n, int block, const f
   BQ_TRY(check_block_args(x, n, block, value, store, values));
   if (n == 0) return BQ_OK;
   uint32_t* out = static_cast<uint32_t*>(values);
-  if (scales_in == nullptr)
-    return value == BQ_Q8S ? launch_block<4, true>(x, n, block, out, scales_out, nullptr, sdt, st)
-                           : launch_block<8, true>(x, n, block, out, scales_out, nullptr, sdt, st);
-  return value == BQ_Q8S ? launch_block<4, false>(x, n, block, out, nullptr, scales_in, sdt, st)
-                         : launch_block<8, false>(x, n, block, out, nullptr, scales_in, sdt, st);
+  if (scales_in == nullptr) return launch_block_for<true>(value, x, n, block, out, scales_out, nullptr, sdt, st);
+  return launch_block_for<false>(value, x, n, block, out, nullptr, scales_in, sdt, st);
 }
 
 // quantize_dynamic of a two-level run-block scheme in one pass over x, given the per-tensor scale.
@@ -1012,9 +1025,8 @@ bq_status launch_quantize_run_block_two_level(const float* x, size_t n, int bloc
                                               float* scales_out, int value, int store, void* values, int sdt, hipStream_t st) {
   BQ_TRY(check_block_args(x, n, block, value, store, values));
   if (n == 0) return BQ_OK;
-  uint32_t* out = static_cast<uint32_t*>(values);
-  return value == BQ_Q8S ? launch_block<4, true, true>(x, n, block, out, scales_out, global, sdt, st, stored_out)
-                         : launch_block<8, true, true>(x, n, block, out, scales_out, global, sdt, st, stored_out);
+  return launch_block_for<true, true>(value, x, n, block, static_cast<uint32_t*>(values), scales_out, global, sdt, st,
+                                      stored_out);
 }
 
 }  // namespace bq

@@ -86,7 +86,7 @@ static bq_status check_scheme(const bq_scheme& s, const size_t* shape, int rank,
   if (rank < 1 || rank > BQ_MAX_RANK) BQ_FAIL(BQ_ERR_SHAPE, "rank %d outside 1..%d", rank, BQ_MAX_RANK);
   BQ_TRY(check_shape_size(shape, rank));
   if (!value_supported(s.value))
-    BQ_FAIL(BQ_ERR_UNSUPPORTED_SCHEME, "Quantization not supported for value %d (Q8S, Q4S and Q2S are)", s.value);
+    BQ_FAIL(BQ_ERR_UNSUPPORTED_SCHEME, "Quantization not supported for value %d (Q8S, Q4S, Q2S, Q8F, Q4F and Q2F are)", s.value);
   if (s.scale_dtype > BQ_SCALE_UE4M3)
     BQ_FAIL(BQ_ERR_UNSUPPORTED_SCHEME, "scale dtype %d is not supported (f32, f16, bf16 and ue4m3 are)", s.scale_dtype);
   if (s.level != BQ_LEVEL_TENSOR && s.level != BQ_LEVEL_BLOCK)
@@ -94,7 +94,7 @@ static bq_status check_scheme(const bq_scheme& s, const size_t* shape, int rank,
   if (s.tensor_scale > 1 || (s.tensor_scale && s.level != BQ_LEVEL_BLOCK))
     BQ_FAIL(BQ_ERR_UNSUPPORTED_SCHEME, "a per-tensor scale on top (tensor_scale = %d) goes with block scales, as f32", s.tensor_scale);
   if (s.store == BQ_STORE_NATIVE) {
-    if (s.value != BQ_Q8S) BQ_FAIL(BQ_ERR_UNSUPPORTED_SCHEME, "Can't store native sub-byte values");
+    if (value_bits(s.value) != 8) BQ_FAIL(BQ_ERR_UNSUPPORTED_SCHEME, "Can't store native sub-byte values");
   } else if (s.store == BQ_STORE_PACKED_U32) {
     if (storable && shape[rank - 1] % static_cast<size_t>(num_quants(s.value)))
       BQ_FAIL(BQ_ERR_SHAPE, "Can't store in u32: last dim %zu is not a multiple of %d", shape[rank - 1],
@@ -1372,7 +1372,7 @@ static bq_status q_gather_impl(const bq_tensor* t, const int32_t* axes, const ui
   // words is stored natively instead of being refused (the reference's CPU backend keeps one i8 per
   // value whatever the store says and permutes freely: ops/quantize.rs:406-431 of its tests ends
   // with a last dim of 2). Sub-byte values have no native store: those results are refused.
-  if (scheme.store == BQ_STORE_PACKED_U32 && scheme.value == BQ_Q8S && new_shape[rank - 1] % 4 != 0)
+  if (scheme.store == BQ_STORE_PACKED_U32 && value_bits(scheme.value) == 8 && new_shape[rank - 1] % 4 != 0)
     scheme.store = BQ_STORE_NATIVE;
   bq_tensor* q = nullptr;
   BQ_TRY(new_quantized(t->dev, scheme, new_shape, rank, &q));  // also: "Can't store in u32" for the new last dim

@@ -2,7 +2,7 @@
 
 `QuantScheme` mirrors cubecl_common::quant::scheme::QuantScheme as burn re-exports it
 (crates/burn-std/src/tensor/quantization.rs:4-6), restricted to what this backend implements:
-symmetric Q8S / Q4S / Q2S values, per-tensor or per-block scales stored as f32, f16, bf16 or ue4m3, an
+symmetric Q8S / Q4S / Q2S and full-range Q8F / Q4F / Q2F values, per-tensor or per-block scales stored as f32, f16, bf16 or ue4m3, an
 optional f32 per-tensor scale on top of block scales (two-level), Native or PackedU32(0) store.
 """
 from __future__ import annotations
@@ -18,12 +18,17 @@ class QuantValue(IntEnum):
     Q8S = _lib.Q8S
     Q4S = _lib.Q4S
     Q2S = _lib.Q2S   # ternary: -1, 0, +1
+    Q8F = _lib.Q8F   # full range: -128..127 (the value of the reference's QuantScheme::default())
+    Q4F = _lib.Q4F   # -8..7
+    Q2F = _lib.Q2F   # -2..1
 
     def range(self) -> Tuple[float, float]:
-        return {QuantValue.Q8S: (-127.0, 127.0), QuantValue.Q4S: (-7.0, 7.0), QuantValue.Q2S: (-1.0, 1.0)}[self]
+        return {QuantValue.Q8S: (-127.0, 127.0), QuantValue.Q4S: (-7.0, 7.0), QuantValue.Q2S: (-1.0, 1.0),
+                QuantValue.Q8F: (-128.0, 127.0), QuantValue.Q4F: (-8.0, 7.0), QuantValue.Q2F: (-2.0, 1.0)}[self]
 
     def size_bits(self) -> int:
-        return {QuantValue.Q8S: 8, QuantValue.Q4S: 4, QuantValue.Q2S: 2}[self]
+        return {QuantValue.Q8S: 8, QuantValue.Q4S: 4, QuantValue.Q2S: 2,
+                QuantValue.Q8F: 8, QuantValue.Q4F: 4, QuantValue.Q2F: 2}[self]
 
 
 class QuantStore(IntEnum):
@@ -45,8 +50,10 @@ class ScaleDtype(IntEnum):
 @dataclass(frozen=True)
 class QuantScheme:
     """value / level (block None = per tensor) / store / scale dtype / per-tensor scale on top of
-    block scales. `QuantScheme()` is the reference default: Q8S, per-tensor, PackedU32(0), f32
-    scales."""
+    block scales. `QuantScheme()` is per-tensor, PackedU32(0), f32 scales like the reference's
+    default, with Q8S values; the reference's own default value is defined in a crate outside its
+    tree and is Q8F according to crates/burn-backend-tests/tests/cubecl/quantization/slice.rs:37-38:
+    pass `value=QuantValue.Q8F` (or `.with_value`) for that."""
 
     value: QuantValue = QuantValue.Q8S
     block: Optional[Tuple[int, ...]] = None

@@ -51,14 +51,18 @@ enum {
 /* DType of a handle. BQ_QFLOAT carries a bq_scheme, like DType::QFloat(scheme). */
 enum { BQ_F32 = 0, BQ_BF16 = 1, BQ_QFLOAT = 2 };
 
-/* QuantValue, QuantStore, quantization level. Only symmetric signed integers are implemented
- * (cubecl_common::quant::scheme, re-exported at crates/burn-std/src/tensor/quantization.rs:4-6).
+/* QuantValue, QuantStore, quantization level (cubecl_common::quant::scheme, re-exported at
+ * crates/burn-std/src/tensor/quantization.rs:4-6). The signed-integer values are implemented:
+ * symmetric Q8S (-127,127), Q4S (-7,7), Q2S (-1,1), and full-range Q8F (-128,127) -- the value of
+ * QuantScheme::default() -- Q4F (-8,7), Q2F (-2,1). A full-range value differs from its symmetric
+ * twin in the quantizer only: scale = 2 absmax / (b - a) with b - a = 255 / 15 / 3, clamp to [a, b];
+ * bits, packing, dequantize and q_matmul are the same.
  * Q2S is the ternary value type of BitNet-style weights (-1, 0, +1; 16 per u32, PackedU32 only):
  * quantize / dequantize / layout ops through the general kernels, and q_matmul's multiply-free
  * path for an f32 lhs times a per-tensor Q2S [K, N] weight
- * (crates/burn-ndarray/src/ops/qtensor.rs:431-517); every other Q2S product dequantizes first, as
- * the reference does. The bqk_ kernel-level entry points take Q8S and Q4S. */
-enum { BQ_Q8S = 0, BQ_Q4S = 1, BQ_Q2S = 2 };
+ * (crates/burn-ndarray/src/ops/qtensor.rs:431-517); every other 2-bit product dequantizes first, as
+ * the reference does. The bqk_ kernel-level entry points take the 8- and 4-bit values. */
+enum { BQ_Q8S = 0, BQ_Q4S = 1, BQ_Q2S = 2, BQ_Q8F = 3, BQ_Q4F = 4, BQ_Q2F = 5 };
 enum { BQ_LEVEL_TENSOR = 0, BQ_LEVEL_BLOCK = 1 };
 enum { BQ_STORE_NATIVE = 0, BQ_STORE_PACKED_U32 = 1 };
 /* ScaleDtype. F16 / BF16 / UE4M3: the quantizer divides by the scale rounded UP to the scale dtype
@@ -70,7 +74,7 @@ enum { BQ_SCALE_F32 = 0, BQ_SCALE_F16 = 1, BQ_SCALE_BF16 = 2, BQ_SCALE_UE4M3 = 3
  * trailing dims (BlockSize::to_dim_vec pads the leading dims with 1). PackedU32 always packs
  * the innermost dim (PackedU32(0)). */
 typedef struct bq_scheme {
-  uint8_t value;       /* BQ_Q8S | BQ_Q4S | BQ_Q2S */
+  uint8_t value;       /* BQ_Q8S | BQ_Q4S | BQ_Q2S | BQ_Q8F | BQ_Q4F | BQ_Q2F */
   uint8_t level;       /* BQ_LEVEL_TENSOR | BQ_LEVEL_BLOCK */
   uint8_t store;       /* BQ_STORE_NATIVE (Q8S only) | BQ_STORE_PACKED_U32 */
   uint8_t scale_dtype; /* BQ_SCALE_F32 | BQ_SCALE_F16 | BQ_SCALE_BF16 | BQ_SCALE_UE4M3 */

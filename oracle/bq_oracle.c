@@ -17,12 +17,18 @@
 
 /* QuantValue::range() lives in cubecl-common (not vendored in the burn tree). Q8S = (-127,127)
  * is fixed by burn-ndarray/src/ops/quantization.rs:164-177; Q4S = (-7,7) by the packed vector in
- * burn-std/src/tensor/quantization.rs:581-602. */
+ * burn-std/src/tensor/quantization.rs:581-602; Q8F = (-128,127) by burn-flex/src/ops/qtensor.rs:665-692
+ * ("Q8F range: [-128, 127], so range = 255", scale = 2 * 7.5 / 255). Q4F = (-8,7) and Q2F = (-2,1)
+ * are the same rule ("full-range", burn-book/src/performance/quantization.md:125-130) at 4 and 2 bits:
+ * PARITY UNPINNED, no reference-held number covers them. */
 int bqo_value_range(int value, float* a, float* b) {
   switch (value) {
     case BQO_Q8S: *a = -127.0f; *b = 127.0f; return 0;
     case BQO_Q4S: *a = -7.0f; *b = 7.0f; return 0;
     case BQO_Q2S: *a = -1.0f; *b = 1.0f; return 0;
+    case BQO_Q8F: *a = -128.0f; *b = 127.0f; return 0;
+    case BQO_Q4F: *a = -8.0f; *b = 7.0f; return 0;
+    case BQO_Q2F: *a = -2.0f; *b = 1.0f; return 0;
     default: return -1;
   }
 }
@@ -30,9 +36,9 @@ int bqo_value_range(int value, float* a, float* b) {
 /* QuantValue::size_bits(), call site burn-std/src/tensor/quantization.rs:520. */
 int bqo_size_bits(int value) {
   switch (value) {
-    case BQO_Q8S: return 8;
-    case BQO_Q4S: return 4;
-    case BQO_Q2S: return 2;
+    case BQO_Q8S: case BQO_Q8F: return 8;
+    case BQO_Q4S: case BQO_Q4F: return 4;
+    case BQO_Q2S: case BQO_Q2F: return 2;
     default: return -1;
   }
 }
@@ -307,7 +313,7 @@ int bqo_decode(const uint8_t* bytes, size_t len, const size_t* shape, int rank,
   size_t split = len - 4 * np;
   memcpy(scales_out, bytes + split, 4 * np);
   size_t n = num_elements(shape, rank);
-  if (s->store == BQO_STORE_NATIVE || s->value == BQO_Q8S) {
+  if (s->store == BQO_STORE_NATIVE || bqo_size_bits(s->value) == 8) {
     /* 8-bit values read back as i8 whatever the store (:329-333); a padded packed line only
      * exists when the innermost dim is not a multiple of 4, which packed backends refuse. */
     if (s->store == BQO_STORE_NATIVE) {

@@ -10,7 +10,9 @@
  * Every function names the reference source it follows (paths relative to the burn tree).
  *
  * Pinning status (what fixes each function besides this restatement):
- *   bqo_value_range      Q8S (-127,127): known answers in burn-ndarray/src/ops/quantization.rs:164-177;
+ *   bqo_value_range      Q8F (-128,127): burn-flex/src/ops/qtensor.rs:665-692; Q4F (-8,7), Q2F (-2,1): PARITY
+ *                        UNPINNED (the same "full-range" rule, no reference-held number);
+ *                        Q8S (-127,127): known answers in burn-ndarray/src/ops/quantization.rs:164-177;
  *                        Q4S (-7,7): the 16 packed words <-> 128 values vector in
  *                        burn-std/src/tensor/quantization.rs:581-602 (it is quantize(arange(128))).
  *   bqo_compute_range    burn-backend-tests .../quantization/calibration.rs:7-59
@@ -80,14 +82,15 @@ extern "C" {
 
 #define BQO_MAX_RANK 8
 
-enum { BQO_Q8S = 0, BQO_Q4S = 1, BQO_Q2S = 2 }; /* QuantValue (symmetric signed ints only); Q2S = ternary */
+/* QuantValue: symmetric (Q2S = ternary) and full-range signed ints */
+enum { BQO_Q8S = 0, BQO_Q4S = 1, BQO_Q2S = 2, BQO_Q8F = 3, BQO_Q4F = 4, BQO_Q2F = 5 };
 enum { BQO_LEVEL_TENSOR = 0, BQO_LEVEL_BLOCK = 1 };
 enum { BQO_STORE_NATIVE = 0, BQO_STORE_PACKED_U32 = 1 };
 enum { BQO_SCALE_F32 = 0, BQO_SCALE_F16 = 1, BQO_SCALE_BF16 = 2, BQO_SCALE_UE4M3 = 3 };   /* ScaleDtype */
 
 /* Mirrors the fields of cubecl_common::quant::scheme::QuantScheme that this path reads. */
 typedef struct {
-  uint8_t value;       /* BQO_Q8S | BQO_Q4S */
+  uint8_t value;       /* BQO_Q8S .. BQO_Q2F */
   uint8_t level;       /* BQO_LEVEL_* */
   uint8_t store;       /* BQO_STORE_* ; PackedU32 always packs the innermost dim */
   uint8_t block_rank;  /* entries used in block[], aligned to the trailing dims */

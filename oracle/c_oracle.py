@@ -14,7 +14,7 @@ import numpy as np
 _HERE = os.path.dirname(os.path.abspath(__file__))
 _LIB_PATH = os.path.join(_HERE, "libbq_oracle.so")
 
-Q8S, Q4S, Q2S = 0, 1, 2
+Q8S, Q4S, Q2S, Q8F, Q4F, Q2F = 0, 1, 2, 3, 4, 5
 LEVEL_TENSOR, LEVEL_BLOCK = 0, 1
 STORE_NATIVE, STORE_PACKED_U32 = 0, 1
 MAX_RANK = 8

@@ -10,8 +10,9 @@ from __future__ import annotations
 
 import numpy as np
 
-RANGES = {"Q8S": (-127.0, 127.0), "Q4S": (-7.0, 7.0), "Q2S": (-1.0, 1.0)}
-BITS = {"Q8S": 8, "Q4S": 4, "Q2S": 2}
+RANGES = {"Q8S": (-127.0, 127.0), "Q4S": (-7.0, 7.0), "Q2S": (-1.0, 1.0),
+          "Q8F": (-128.0, 127.0), "Q4F": (-8.0, 7.0), "Q2F": (-2.0, 1.0)}
+BITS = {"Q8S": 8, "Q4S": 4, "Q2S": 2, "Q8F": 8, "Q4F": 4, "Q2F": 2}
 
 
 def _block_dims(shape, block):

@@ -18,7 +18,8 @@ import burn_amd as ba  # noqa: E402
 from burn_amd import FloatOps, ModuleOps, QTensorOps, QuantScheme, QuantStore, QuantValue, TensorData  # noqa: E402
 from burn_amd.quantization import ScaleDtype  # noqa: E402
 
-VAL = {QuantValue.Q8S: (co.Q8S, "Q8S"), QuantValue.Q4S: (co.Q4S, "Q4S"), QuantValue.Q2S: (co.Q2S, "Q2S")}
+VAL = {QuantValue.Q8S: (co.Q8S, "Q8S"), QuantValue.Q4S: (co.Q4S, "Q4S"), QuantValue.Q2S: (co.Q2S, "Q2S"),
+       QuantValue.Q8F: (co.Q8F, "Q8F"), QuantValue.Q4F: (co.Q4F, "Q4F"), QuantValue.Q2F: (co.Q2F, "Q2F")}
 
 
 @pytest.fixture(scope="module")
@@ -1041,15 +1042,88 @@ def test_q2s_ternary_matmul_is_the_reference_sum(dev):
     matmul_check(gotb, no.q_matmul_f64(x, qb, sb, [16]))
 
 
+# ------------------------------------------------------------------ full-range values
+
+def test_q8f_reference_case(dev, kats):
+    """crates/burn-flex/src/ops/qtensor.rs:665-692: Q8F spans [-128, 127], scale = 2 * 7.5 / 255,
+    dequantized within 0.1 of the input."""
+    k = kats["quantize_dynamic_q8f"]
+    x = np.float32(k["x"])
+    for store in (QuantStore.Native, QuantStore.PackedU32):
+        xs = x if store == QuantStore.Native else np.concatenate([x, np.float32([0, 0])])   # (whole packed words)
+        tq = QTensorOps.quantize_dynamic(FloatOps.float_from_data(xs, dev), QuantScheme(value=QuantValue.Q8F, store=store))
+        q, s = unpack_blob(QTensorOps.q_into_data(tq))
+        assert abs(float(s.reshape(-1)[0]) - k["expected_scale"]) < k["scale_abs_tol"]
+        assert s.reshape(-1)[0] == np.float32(2 * 7.5) / np.float32(255)
+        assert q[-1 if store == QuantStore.Native else 5] == 127 and q.min() >= -128
+        d = FloatOps.float_into_data(QTensorOps.dequantize(tq))
+        assert np.abs(d[:6] - x).max() < k["dequant_abs_tol"]
+    # the negative end of the range is reached: -absmax / s = -127.5 rounds to -128
+    tq = QTensorOps.quantize_dynamic(FloatOps.float_from_data(-x, dev), QuantScheme(value=QuantValue.Q8F, store=QuantStore.Native))
+    q, _ = unpack_blob(QTensorOps.q_into_data(tq))
+    assert q[5] == -128 and q[0] == 85
+
+
+@pytest.mark.parametrize("value", [QuantValue.Q8F, QuantValue.Q4F, QuantValue.Q2F])
+@pytest.mark.parametrize("block", [None, (32,), (16,), (2, 32), (128,)])
+def test_full_range_values_against_the_oracle(dev, value, block):
+    """quantize_dynamic / quantize / dequantize with full-range values on every kernel route (per
+    tensor, fused run blocks, rectangles), f32 and narrow scales, two-level: bit for bit."""
+    x = awkward((64, 256), 77)
+    x[5, :64] = 0.0
+    scheme = QuantScheme(value=value) if block is None else QuantScheme(value=value).per_block(block)
+    tq, q_ref, s_ref, _ = check_quantize_dynamic(dev, x, scheme)
+    lo, hi = value.range()
+    assert q_ref.min() >= lo and q_ref.max() <= hi and (q_ref.min() == lo or q_ref.max() == hi)
+    if block is not None:   # among many blocks both ends of the range are reached
+        assert q_ref.min() == lo and q_ref.max() == hi
+    if value == QuantValue.Q8F:
+        native = QuantScheme(value=value, store=QuantStore.Native, block=block)
+        check_quantize_dynamic(dev, x, native)
+        check_quantize_dynamic(dev, x.reshape(-1)[: 64 * 256 - 3 if block is None else 64 * 256], native if block is None else
+                               QuantScheme(value=value, store=QuantStore.Native).per_block((32,)))
+    # given scales (every route quantizes against them, zero scales included)
+    given = s_ref.copy().reshape(-1) * np.float32(0.75)
+    given[::5] = 0.0
+    t = QTensorOps.quantize(FloatOps.float_from_data(x, dev), scheme, FloatOps.float_from_data(given, dev))
+    q, s = unpack_blob(QTensorOps.q_into_data(t))
+    assert s.reshape(-1).tobytes() == given.tobytes() and (q == co.quantize(x, oscheme(scheme), given)).all()
+    check_scale_dtype(dev, x, QuantScheme(value=value, block=block, scale_dtype=ScaleDtype.BF16))
+    if block is not None:
+        check_two_level(dev, x, scheme.with_scale_dtype(ScaleDtype.F16).per_tensor(ScaleDtype.F32))
+
+
+@pytest.mark.parametrize("value", [QuantValue.Q8F, QuantValue.Q4F])
+def test_q_matmul_with_full_range_weights(dev, value):
+    """The products read two's complement fields: a weight that uses the extra negative code goes
+    through every kernel family like its symmetric twin."""
+    rng = np.random.default_rng(31)
+    w = (rng.standard_normal((512, 384)) * 0.02).astype(np.float32)
+    w[np.arange(512), rng.integers(0, 384, 512)] = -0.11          # the block minimum: quantized to the lowest code
+    for block in (None, (32,), (128,)):
+        scheme = QuantScheme(value=value) if block is None else QuantScheme(value=value).per_block(block)
+        tw, q_ref, s_ref, wd = check_quantize_dynamic(dev, w, scheme)
+        assert q_ref.min() == value.range()[0]
+        for m, dt in ((1, ba.F32), (2, ba.BF16), (4, ba.F32), (16, ba.F32), (24, ba.BF16), (48, ba.F32), (130, ba.BF16)):
+            xh = rng.standard_normal((m, 512)).astype(np.float32)
+            if dt == ba.BF16:
+                bits = ba.bf16_bits_from_f32(xh)
+                lhs, xd = FloatOps.float_from_data(bits, dev, ba.BF16), ba.f32_from_bf16_bits(bits)
+            else:
+                lhs, xd = FloatOps.float_from_data(xh, dev), xh
+            out = FloatOps.float_into_data(QTensorOps.q_matmul(lhs, tw, out_dtype=ba.F32))
+            matmul_check(out, xd.astype(np.float64) @ wd.astype(np.float64))
+
+
 # ------------------------------------------------------------------ random schemes
 
 def random_scheme_case(rng):
     """A quantizable (shape, scheme, magnitude): value, store, rank 1-4, per tensor or a block of rank
     1-rank with power-of-two extents (whole packed words along the last dim), any scale dtype, the
     two-level form for f16 / ue4m3 block scales."""
-    value = [QuantValue.Q8S, QuantValue.Q4S, QuantValue.Q2S][rng.integers(3)]
-    nq = {QuantValue.Q8S: 4, QuantValue.Q4S: 8, QuantValue.Q2S: 16}[value]
-    store = QuantStore.Native if value == QuantValue.Q8S and rng.integers(2) else QuantStore.PackedU32
+    value = [QuantValue.Q8S, QuantValue.Q4S, QuantValue.Q2S, QuantValue.Q8F, QuantValue.Q4F, QuantValue.Q2F][rng.integers(6)]
+    nq = 32 // value.size_bits()
+    store = QuantStore.Native if nq == 4 and rng.integers(2) else QuantStore.PackedU32
     rank = int(rng.integers(1, 5))
     sdt = [ScaleDtype.F32, ScaleDtype.F16, ScaleDtype.BF16, ScaleDtype.UE4M3][rng.integers(4)]
     block = None
@@ -1073,12 +1147,12 @@ def random_scheme_case(rng):
 
 
 def test_random_schemes_against_the_oracle(dev):
-    """200 seeded cases over the whole scheme space: quantize_dynamic's blob, the dequantized floats
+    """300 seeded cases over the whole scheme space: quantize_dynamic's blob, the dequantized floats
     and the blob round trip bit for bit, then one layout op (swap / permute / flip) on the result,
     whose dequantized values must be the same permutation of the source's."""
     rng = np.random.default_rng(20240607)
     seen = set()
-    for case in range(200):
+    for case in range(300):
         shape, scheme, mag = random_scheme_case(rng)
         x = (rng.standard_normal(shape) * mag).astype(np.float32)
         if rng.integers(5) == 0:
@@ -1098,7 +1172,7 @@ def test_random_schemes_against_the_oracle(dev):
         rank = len(shape)
         axes = [int(a) for a in rng.permutation(rank)]
         nq = tq.scheme.num_quants()
-        if rank > 1 and (scheme.store == QuantStore.Native or scheme.value == QuantValue.Q8S or shape[axes[-1]] % nq == 0):
+        if rank > 1 and (nq == 4 or shape[axes[-1]] % nq == 0):
             tp = QTensorOps.q_permute(tq, axes)
             got = FloatOps.float_into_data(QTensorOps.dequantize(tp))
             assert got.tobytes() == np.ascontiguousarray(np.transpose(d, axes)).tobytes(), f"{label}: permute {axes}"
@@ -1106,7 +1180,7 @@ def test_random_schemes_against_the_oracle(dev):
         if scheme.block is None:   # (a flip keeps block scales in place: only per-tensor values commute with it)
             got = FloatOps.float_into_data(QTensorOps.dequantize(QTensorOps.q_flip(tq, fl)))
             assert got.tobytes() == np.ascontiguousarray(np.flip(d, fl)).tobytes(), f"{label}: flip {fl}"
-    assert len(seen) >= 36   # of the 40 (value, store) x (level, scale dtype, two-level) combinations
+    assert len(seen) >= 60   # of the 80 (value, store) x (level, scale dtype, two-level) combinations
 
 
 def test_random_matmuls_against_float64(dev):
@@ -1118,8 +1192,8 @@ def test_random_matmuls_against_float64(dev):
 
     def family_case():
         """Weights shaped for the fused kernels: whole 128-column groups, K in 32-row steps (or not)."""
-        value = [QuantValue.Q8S, QuantValue.Q4S][rng.integers(2)]
-        store = QuantStore.Native if value == QuantValue.Q8S and rng.integers(3) == 0 else QuantStore.PackedU32
+        value = [QuantValue.Q8S, QuantValue.Q4S, QuantValue.Q8F, QuantValue.Q4F][rng.integers(4)]
+        store = QuantStore.Native if value.size_bits() == 8 and rng.integers(3) == 0 else QuantStore.PackedU32
         n = int([128, 256, 384, 640, 1024, 96, 48][rng.integers(7)])
         k = int([32, 64, 96, 256, 512, 1000, 40][rng.integers(7)])
         block = [None, (32,), (64,), (128,), (16,), (8,)][rng.integers(6)]
@@ -1147,6 +1221,11 @@ def test_random_matmuls_against_float64(dev):
             if scheme.block is not None and len(scheme.block) >= 2:
                 kb = scheme.block[-2]
             shape = shape[:-2] + (shape[-2] * int(rng.integers(2, 9)) * (32 // np.gcd(32, kb) if rng.integers(2) else 1),) + shape[-1:]
+            # (K stays at 2048 and below: on the kernels that round to bf16 the error is 2.3e-3 of the
+            # output's rms, and with these inputs the elementwise rule's absolute 1e-2 is 4.8 sigma
+            # there; at K = 6144 it is 2.8 sigma and a few outputs in a thousand pass it)
+            while shape[-2] > 2048 and shape[-2] % 2 == 0:
+                shape = shape[:-2] + (shape[-2] // 2,) + shape[-1:]
         rank = len(shape)
         w = (rng.standard_normal(shape) * 0.02).astype(np.float32)
         tw = QTensorOps.quantize_dynamic(FloatOps.float_from_data(w, dev), scheme)

@@ -15,7 +15,7 @@ def f32(v):
 
 
 def scheme(value="Q8S", block=None, store=co.STORE_NATIVE):
-    return co.Scheme.make({"Q8S": co.Q8S, "Q4S": co.Q4S}[value], block, store)
+    return co.Scheme.make({"Q8S": co.Q8S, "Q4S": co.Q4S, "Q2S": co.Q2S, "Q8F": co.Q8F, "Q4F": co.Q4F, "Q2F": co.Q2F}[value], block, store)
 
 
 # ---------------------------------------------------------------- quantize / dequantize KATs
@@ -73,6 +73,21 @@ def test_quantize_dynamic_int8(kats):
     assert s.tobytes() == f32([k["expected_scale"]]).tobytes()
     qn, sn = no.quantize_dynamic(f32(k["x"]))
     assert qn.tolist() == k["expected_q"] and sn.tobytes() == s.tobytes()
+
+
+def test_quantize_dynamic_q8f(kats):
+    """Full-range int8 as burn-flex pins it: range [-128, 127], scale = 2 * 7.5 / 255, dequantized
+    within 0.1; the absmax element lands on 127.5 -> 128 -> clamped to 127, its negation on -128."""
+    k = kats["quantize_dynamic_q8f"]
+    x = f32(k["x"])
+    for q, s in (co.quantize_dynamic(x, scheme("Q8F")), no.quantize_dynamic(x, "Q8F")):
+        assert abs(float(s.reshape(-1)[0]) - k["expected_scale"]) < k["scale_abs_tol"]
+        assert s.reshape(-1)[0] == F32(2 * 7.5) / F32(255)
+        assert q.tolist() == [-85, -43, 0, 43, 85, 127]
+        assert np.abs(q.astype(np.float32) * s.reshape(-1)[0] - x).max() < k["dequant_abs_tol"]
+    q, _ = co.quantize_dynamic(-x, scheme("Q8F"))
+    assert q.tolist() == [85, 43, 0, -43, -85, -128]
+    assert no.RANGES["Q8F"] == tuple(float(v) for v in k["range"])
 
 
 def test_quantize_dynamic_arange32_times_10(kats, approx):
@@ -308,7 +323,7 @@ def test_block_of_matches_reshape_bruteforce():
         assert co.dequantize(qc, sch, sc).tobytes() == no.dequantize(qn, sn, block).tobytes()
 
 
-@pytest.mark.parametrize("value", ["Q8S", "Q4S"])
+@pytest.mark.parametrize("value", ["Q8S", "Q4S", "Q8F", "Q4F", "Q2F"])
 @pytest.mark.parametrize("block", [None, [32]])
 def test_c_and_numpy_restatements_agree(value, block):
     rng = np.random.default_rng(11)
