@@ -76,7 +76,7 @@ enum { BQ_SCALE_F32 = 0, BQ_SCALE_F16 = 1, BQ_SCALE_BF16 = 2, BQ_SCALE_UE4M3 = 3
 typedef struct bq_scheme {
   uint8_t value;       /* BQ_Q8S | BQ_Q4S | BQ_Q2S | BQ_Q8F | BQ_Q4F | BQ_Q2F */
   uint8_t level;       /* BQ_LEVEL_TENSOR | BQ_LEVEL_BLOCK */
-  uint8_t store;       /* BQ_STORE_NATIVE (Q8S only) | BQ_STORE_PACKED_U32 */
+  uint8_t store;       /* BQ_STORE_NATIVE (8-bit values only) | BQ_STORE_PACKED_U32 */
   uint8_t scale_dtype; /* BQ_SCALE_F32 | BQ_SCALE_F16 | BQ_SCALE_BF16 | BQ_SCALE_UE4M3 */
   uint8_t block_rank;
   uint8_t tensor_scale; /* block level only: 1 = an f32 per-tensor scale on top of the block scales (below) */
