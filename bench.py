@@ -552,6 +552,21 @@ def run_next(ba, dev, steps, warmup, cpu):
                                        "relative to an f32 per-tensor scale (two launches more: the largest scale, the split)",
                            "parity": "blob and dequantized floats bit-exact vs CPU oracle on a 256-row tensor of the same data", **sd}
 
+    # ---- the full-range value of the reference's default scheme --------------------------------------
+    osch_f = co.Scheme.make(co.Q8F, [32], co.STORE_PACKED_U32)
+    scheme_f = QuantScheme(value=QuantValue.Q8F).per_block((32,))
+    tq = QTensorOps.quantize_dynamic(FloatOps.float_from_data(small, dev), scheme_f)
+    q_ref, s_ref = co.quantize_dynamic(small, osch_f)
+    if QTensorOps.q_into_data(tq).bytes.tobytes() != co.encode(q_ref, osch_f, s_ref).tobytes() or \
+            FloatOps.float_into_data(QTensorOps.dequantize(tq)).tobytes() != co.dequantize(q_ref, osch_f, s_ref).tobytes():
+        raise ParityError("Q8F: blob or dequantized floats differ from the CPU oracle's")
+    t_q = graph_ms(dev, lambda: [QTensorOps.quantize_dynamic(xs[i % 5], scheme_f) for i in range(10)], 10, steps, warmup)
+    b = 4 * nel + nel + 4 * nel // 32
+    out["full_range"] = {"workload": "C2's tensor, Q8F (-128..127, span 255) block-32 PackedU32, f32 scales: quantize_dynamic",
+                         "parity": "blob and dequantized floats bit-exact vs CPU oracle on a 256-row tensor of the same data",
+                         "quantize_dynamic": {"ms": t_q, "GB/s": b / t_q / 1e6, "frac_hbm": b / t_q / 1e6 / HBM_PEAK_GBS}, "bytes": b}
+    dev.trim()
+
     # ---- layout ops on a packed tensor -------------------------------------------------------------
     scheme = QuantScheme().per_block((32,))
     tq_small = QTensorOps.quantize_dynamic(FloatOps.float_from_data(small, dev), scheme)
