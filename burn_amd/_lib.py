@@ -99,6 +99,7 @@ SIGNATURES = {
     "bq_float_empty": (_i32, [_vp, _i32, _psz, _i32, _pvp]),
     "bq_float_from_device_ptr": (_i32, [_vp, _vp, _i32, _psz, _i32, _pvp]),
     "bq_float_matmul": (_i32, [_vp, _vp, _pvp]),
+    "bq_scheme_supported": (_i32, [_ps]),
     "bq_quantized_data_len": (_i32, [_ps, _psz, _i32, _psz]),
     "bq_q_from_data": (_i32, [_vp, _vp, _sz, _psz, _i32, _ps, _pvp]),
     "bq_q_into_data": (_i32, [_vp, _vp, _sz, _psz]),

@@ -591,6 +591,31 @@ extern "C" bq_status bq_float_from_device_ptr(bq_device* dev, void* device_ptr, 
 }
 
 // ================================================================================ wire format
+extern "C" bq_status bq_scheme_supported(const bq_scheme* scheme) {
+  BQ_NOTNULL(scheme);
+  const bq_scheme& s = *scheme;
+  // the shape-independent half of check_scheme: a shape of block extents satisfies the other half
+  size_t shape[BQ_MAX_RANK];
+  int rank = 1;
+  if (s.level == BQ_LEVEL_BLOCK) {
+    if (s.block_rank < 1 || s.block_rank > BQ_MAX_RANK)
+      BQ_FAIL(BQ_ERR_UNSUPPORTED_SCHEME, "block of rank %d (1..%d are supported)", s.block_rank, BQ_MAX_RANK);
+    rank = s.block_rank;
+    for (int d = 0; d < rank; ++d) shape[d] = s.block[d];
+    if (s.block[rank - 1] == 0) BQ_FAIL(BQ_ERR_UNSUPPORTED_SCHEME, "a block extent of 0");
+  } else {
+    shape[0] = 1;
+  }
+  shape[rank - 1] *= 16;  // (whole packed words along the last dim for every value width)
+  bq_status rc = check_scheme(s, shape, rank);
+  if (rc != BQ_OK) return rc == BQ_ERR_SHAPE ? BQ_ERR_UNSUPPORTED_SCHEME : rc;
+  // quantizable: normalize_scales needs block scales that f16's range holds
+  if (s.tensor_scale && s.scale_dtype != BQ_SCALE_F16 && s.scale_dtype != BQ_SCALE_UE4M3)
+    BQ_FAIL(BQ_ERR_UNSUPPORTED_SCHEME,
+            "block scales of this dtype reach f32's range, which a per-tensor scale cannot absorb (f16 and ue4m3 block scales can)");
+  return BQ_OK;
+}
+
 extern "C" bq_status bq_quantized_data_len(const bq_scheme* scheme, const size_t* shape, int32_t rank,
                                            size_t* len_out) {
   BQ_NOTNULL(scheme);

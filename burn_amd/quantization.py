@@ -91,6 +91,15 @@ class QuantScheme:
     def with_scale_dtype(self, scale_dtype: ScaleDtype) -> "QuantScheme":
         return replace(self, scale_dtype=scale_dtype)
 
+    def supported(self) -> bool:
+        """What `Backend::dtype_usage(DType::QFloat(self))` answers: the library implements the
+        scheme, and it is `quantizable` (crates/burn-std/src/tensor/quantization.rs:113-128)."""
+        try:
+            c = self.to_c()
+        except ValueError:
+            return False
+        return _lib.lib().bq_scheme_supported(_lib.C.byref(c)) == _lib.OK
+
     def num_quants(self) -> int:
         return 32 // self.value.size_bits() if self.store == QuantStore.PackedU32 else 1
 

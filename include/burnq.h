@@ -188,6 +188,16 @@ bq_status bq_float_matmul(const bq_tensor* lhs, const bq_tensor* rhs, bq_tensor*
  * crates/burn-backend/src/backend/ops/qtensor.rs:123-1324; the CPU semantics these reproduce bit
  * for bit are burn-ndarray's (crates/burn-ndarray/src/ops/qtensor.rs, ops/quantization.rs). */
 
+/* Whether this backend takes tensors of `scheme`, whatever their shape: what the binding answers
+ * Backend::dtype_usage(DType::QFloat(scheme)) with (pattern: crates/burn-ndarray/src/backend.rs:98-119).
+ * The values, stores and levels this library implements, under the reference's `quantizable` rule
+ * (crates/burn-std/src/tensor/quantization.rs:113-128): a scale dtype with a round-up rule, and for a
+ * two-level scheme block scales whose largest value does not exceed f16's (F16, UE4M3) under an f32
+ * per-tensor scale. BQ_OK, or BQ_ERR_UNSUPPORTED_SCHEME with the reason in bq_last_error().
+ * (bq_quantize_two_level with given parameters is laxer about the block scale dtype, as the
+ * reference's quantize is; this is the answer for schemes to quantize dynamically against.) */
+bq_status bq_scheme_supported(const bq_scheme* scheme);
+
 /* Bytes of the TensorData blob for `shape` under `scheme`: values || block scales, dense.
  * quantized_data_len -- crates/burn-std/src/tensor/quantization.rs:400-407. */
 bq_status bq_quantized_data_len(const bq_scheme* scheme, const size_t* shape, int32_t rank,

@@ -116,6 +116,33 @@ def test_data_len_refuses_what_q_from_data_would_refuse():
     assert status(bad, (4, 64)) == _lib.ERR_UNSUPPORTED_SCHEME
 
 
+def test_scheme_supported_follows_the_reference_quantizable_rule():
+    """bq_scheme_supported on the cases of the reference's own test of `quantizable`
+    (crates/burn-std/src/tensor/quantization.rs:713-744), and on what this library does not store."""
+    from burn_amd.quantization import QuantStore, QuantValue
+    base = QuantScheme()
+    assert base.supported() and base.with_value(QuantValue.Q8F).supported()
+    assert base.per_block((4,), ScaleDtype.F16).supported()
+    assert base.per_block((4,), ScaleDtype.UE4M3).per_tensor(ScaleDtype.F32).supported()
+    assert base.per_block((4,), ScaleDtype.F16).per_tensor(ScaleDtype.F32).supported()
+    # block scales reaching f32's range leave the per-tensor scale subnormal
+    assert not base.per_block((4,), ScaleDtype.F32).per_tensor(ScaleDtype.F32).supported()
+    assert not base.per_block((4,), ScaleDtype.BF16).per_tensor(ScaleDtype.F32).supported()
+    assert b"cannot absorb" in _lib.lib().bq_last_error()
+    with pytest.raises(ValueError):          # a per-tensor scale narrower than f32 (refused where the scheme is built)
+        base.per_block((4,), ScaleDtype.UE4M3).per_tensor(ScaleDtype.BF16)
+    # every value, packed; native only at 8 bits; rectangle blocks; unknown codes
+    for v in QuantValue:
+        assert QuantScheme(value=v).supported() and QuantScheme(value=v).per_block((2, 32)).supported()
+        assert QuantScheme(value=v, store=QuantStore.Native).supported() == (v.size_bits() == 8)
+    c = base.to_c()
+    c.value = 9
+    assert _lib.lib().bq_scheme_supported(C.byref(c)) == _lib.ERR_UNSUPPORTED_SCHEME
+    c = base.to_c()
+    c.scale_dtype = 7                        # (a dtype without a round-up rule, like ue8m0 there)
+    assert _lib.lib().bq_scheme_supported(C.byref(c)) == _lib.ERR_UNSUPPORTED_SCHEME
+
+
 def test_shapes_whose_sizes_would_overflow_are_refused():
     """Element and byte counts are products of caller-supplied dims: a shape past 2^44 elements is
     refused before anything is multiplied (no wrapped-around allocation size)."""
