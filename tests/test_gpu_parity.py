@@ -630,10 +630,18 @@ def test_hip_graph_replays_match_eager(dev):
     a64 = FloatOps.float_from_data(ba.bf16_bits_from_f32(rng.standard_normal((64, 512)).astype(np.float32)), dev, ba.BF16)
     bias = FloatOps.float_from_data(rng.standard_normal(256).astype(np.float32), dev)
 
+    wt = QTensorOps.quantize_dynamic(FloatOps.float_from_data(awkward((512, 256), 4, outliers=False), dev),
+                                     QuantScheme(value=QuantValue.Q2S))
+
     def step():
         qt = QTensorOps.quantize_dynamic(x, QuantScheme(store=QuantStore.Native))
         qb = QTensorOps.quantize_dynamic(x, QuantScheme(value=QuantValue.Q4S).per_block((32,)))
-        return (qt, qb, QTensorOps.dequantize(qt), QTensorOps.dequantize(qb),
+        # two-level scales (absmax, per-tensor scale, split block kernel), a full-range value,
+        # the tiled transpose with its scale gather, the ternary product
+        q2 = QTensorOps.quantize_dynamic(x, QuantScheme().per_block((32,), ScaleDtype.UE4M3).per_tensor(ScaleDtype.F32))
+        qf = QTensorOps.quantize_dynamic(x, QuantScheme(value=QuantValue.Q8F).per_block((64,)))
+        return (qt, qb, q2, qf, QTensorOps.dequantize(q2), QTensorOps.q_swap_dims(qf, 0, 1), QTensorOps.q_matmul(a4, wt),
+                QTensorOps.dequantize(qt), QTensorOps.dequantize(qb),
                 QTensorOps.q_matmul(a, w), QTensorOps.q_matmul(a4, w),
                 # matrix cores over split activations; tiled kernel with split K; bias epilogues
                 QTensorOps.q_matmul(a16, w), ModuleOps.linear(a16, w, bias),
