@@ -5,15 +5,18 @@
 // scale per tensor or per run of `block` values along N (scales[k][n / block]). The reference
 // (crates/burn-ndarray/src/ops/qtensor.rs:223-267) materialises dequantize(W) and calls an sgemm;
 // here the dequantize is fused into the operand path:
-//   * decode (f32 lhs, M <= 4): a q-GEMV that unpacks in registers, split over K; HBM bound.
-//   * f32 lhs, 5 <= M <= 32: the split-activation kernel of qsplit.hip (bf16 matrix cores, exact
-//     int8 weights, activations x scale as two bf16 terms); the weight layouts it does not take
-//     fall back to the decode kernel (M <= 8), the FP32-matrix kernel of qskinny.hip, or the
-//     general q-GEMV below.
-//   * bf16 lhs with M <= 32: the same split-activation kernel (bf16 x scale needs the two terms
-//     as well). Other layouts: the bf16 kernel of qskinny.hip (M <= 32).
+//   * decode (f32 lhs: M <= 3 on 8-bit weights, M <= 2 on 4-bit ones; bf16 lhs: M <= 2): a q-GEMV
+//     that unpacks in registers, split over K; HBM bound.
+//   * from there up to M = 32: the split-activation kernel of qsplit.hip (bf16 matrix cores, exact
+//     integer weights, activations x scale as two bf16 terms); the weight layouts it does not take
+//     fall back to the decode kernel (M <= 8), the kernels of qskinny.hip, or the general q-GEMV
+//     below.
 //   * prefill: packed words + scales -> registers -> bf16 in LDS -> v_mfma_f32_32x32x16_bf16,
-//     f32 accumulation.
+//     f32 accumulation (qgemm.hip).
+// Also here: the fixed-order reduction of the K slices, the f32 matrix-core GEMM of the general
+// path (operands that are dequantized first), the multiply-free product of ternary weights, and
+// the allocation-free entry point. Full-range values (Q8F, Q4F) are two's complement fields like
+// their symmetric twins and take the same kernels.
 #include <algorithm>
 
 #include <type_traits>

@@ -1,6 +1,6 @@
-// Small-batch q_matmul on the bf16 matrix cores (gfx950) at better than bf16 accuracy, M <= 16:
-// out[M,N] = X[M,K] x dequantize(W[K,N]), X f32 or bf16, W Q8S or Q4S with one scale per 32
-// columns (or per tensor).
+// Small-batch q_matmul on the bf16 matrix cores (gfx950) at better than bf16 accuracy, M <= 32:
+// out[M,N] = X[M,K] x dequantize(W[K,N]), X f32 or bf16, W 8- or 4-bit with one scale per 32, 64
+// or 128 columns (or per tensor).
 //
 // Same operation as the other q_matmul kernels (QTensorOps::q_matmul,
 // crates/burn-backend/src/backend/ops/qtensor.rs:498-544; reference path
