@@ -1,4 +1,4 @@
-"""Build-time check of the prefill q-GEMM's hand-managed global loads.
+"""Build-time checks of the prefill q-GEMM's hand-managed global loads and matrix instructions.
 
 qgemm.hip issues its global loads through inline asm, so the compiler does not know that the
 destination registers are written asynchronously: only the kernel's own `s_waitcnt vmcnt(N)`
@@ -8,6 +8,11 @@ silently corrupt data. This module scans the generated ISA of every `qgemm_kerne
 it replays the instruction stream (prologue, three trips of the main loop, epilogue) with an
 in-order queue of outstanding loads, retires loads at every `s_waitcnt vmcnt(N)`, and reports any
 instruction that reads or overwrites a register whose load is still outstanding.
+
+The matrix instructions are inline asm as well, so the compiler's hazard recognizer does not see
+them either: a vector instruction may read an accumulator only kMfmaDrain wait states after the
+last MFMA that wrote it (the kernel drains with `s_nop`s before it leaves the loop). The same scan
+counts the wait states between every MFMA and the first other instruction that reads its result.
 
     python -m burn_amd.isa_check            # compiles qgemm.hip to ISA and checks it
 """
@@ -22,6 +27,10 @@ import tempfile
 HERE = os.path.dirname(os.path.abspath(__file__))
 
 _REG = re.compile(r"\bv\[(\d+):(\d+)\]|\bv(\d+)\b")
+_ACC = re.compile(r"\ba\[(\d+):(\d+)\]|\ba(\d+)\b")
+# wait states a 16-pass matrix instruction needs before a vector instruction may read its result
+# (one per issued instruction, N + 1 per `s_nop N`); the kernel's drain is 48
+kMfmaDrain = 20
 _LOADS = ("buffer_load", "global_load", "scratch_load")
 _NO_DEST = ("ds_write", "buffer_store", "global_store", "scratch_store", "s_", "v_cmp")
 
@@ -46,6 +55,45 @@ def _kernels(lines):
             yield m.group(1), lines[i:end]
             i = end
         i += 1
+
+
+def _accs(text):
+    out = set()
+    for m in _ACC.finditer(text):
+        if m.group(1):
+            out |= set(range(int(m.group(1)), int(m.group(2)) + 1))
+        else:
+            out.add(int(m.group(3)))
+    return out
+
+
+def check_mfma_drain(seq):
+    """Instructions other than MFMAs that read an accumulator register too soon after the MFMA that
+    wrote it. `seq`: the instruction stream as it executes (the loop unrolled)."""
+    written, hazards = {}, []          # accumulator register -> wait states since its last MFMA
+    for line in seq:
+        line = line.split(";")[0].strip()
+        if not line or line.endswith(":") or line.startswith("."):
+            continue
+        op, _, rest = line.partition(" ")
+        ops = rest.split(",")
+        if op.startswith("v_mfma"):
+            for r in written:
+                written[r] += 1
+            for r in _accs(ops[0]):
+                written[r] = 0
+            continue
+        if op == "s_nop":
+            step = int(rest.strip()) + 1
+        else:
+            step = 1
+            early = [r for r in _accs(",".join(ops[1:]) if not op.startswith(_NO_DEST) else rest)
+                     if written.get(r, kMfmaDrain) < kMfmaDrain]
+            if early:
+                hazards.append((line, sorted(early)))
+        for r in written:
+            written[r] += step
+    return hazards
 
 
 def check_kernel(body):
@@ -91,6 +139,8 @@ def check_kernel(body):
         if is_load:
             pending.append(dst)
             max_out = max(max_out, len(pending))
+    # the matrix instructions' results: the last trip (with its drain) and what follows the loop
+    hazards += check_mfma_drain(body[:hdr] + without_exit_drain(loop) + loop + body[back + 1:])
     return hazards, max_out
 
 
@@ -121,7 +171,8 @@ def compile_and_check(hipcc=None, flags=None):
     if bad:
         msg = "\n".join(f"{k}: {len(h)} finding(s), first: {h[0][0]} (registers {h[0][1]})"
                         for k, (h, _) in bad.items())
-        raise RuntimeError("qgemm.hip: registers of outstanding loads are touched before their wait:\n" + msg)
+        raise RuntimeError("qgemm.hip: a register is touched before its load's wait, or an accumulator is read "
+                           "before its matrix instruction has drained:\n" + msg)
     return report
 
 

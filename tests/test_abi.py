@@ -242,7 +242,13 @@ def test_isa_check_flags_an_unwaited_load(tmp_path):
         "\tv_add_u32_e32 v6, v5, v5\n\ts_waitcnt vmcnt(0)\n\tbuffer_load_dword v5, v1, s[0:3], 0 offen\n" + tail
     younger = head + "\tbuffer_load_dword v5, v1, s[0:3], 0 offen\n\tbuffer_load_dword v7, v1, s[0:3], 0 offen\n" + loop + \
         "\ts_waitcnt vmcnt(1)\n\tv_add_u32_e32 v6, v5, v5\n\tv_mov_b32_e32 v8, v7\n\ts_waitcnt vmcnt(0)\n" + tail
-    for name, text, findings in (("good", good, 0), ("bad", bad, 3), ("younger", younger, 1)):
+    # an accumulator read before its matrix instruction has drained (inline-asm MFMAs are invisible
+    # to the compiler's own hazard recognizer)
+    mfma = "\tv_mfma_f32_32x32x16_bf16 a[0:15], v[2:5], v[6:9], a[0:15]\n"
+    drained = head + loop + mfma + "\ts_nop 15\n\ts_nop 15\n" + tail.replace("\ts_endpgm", "\tv_accvgpr_read_b32 v1, a3\n\ts_endpgm")
+    early = head + loop + mfma + "\ts_nop 3\n" + tail.replace("\ts_endpgm", "\tv_accvgpr_read_b32 v1, a3\n\ts_endpgm")
+    for name, text, findings in (("good", good, 0), ("bad", bad, 3), ("younger", younger, 1), ("drained", drained, 0),
+                                 ("early", early, 1)):
         path = tmp_path / f"{name}.s"
         path.write_text(text)
         report = isa_check.check_listing(str(path))
