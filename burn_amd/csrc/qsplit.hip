@@ -28,9 +28,12 @@
 // A wave owns 4 adjacent blocks (128 columns: a row is 128 bytes of Q8S or 64 of Q4S) and a run
 // of k rows; the 8 waves of a workgroup are 4 such column groups x 2 halves of the workgroup's K
 // slice, whose activations sit in LDS. The weights are loaded as whole rows (16 bytes per lane)
-// and handed to the lanes that multiply them through a small LDS slot private to the wave. The
-// two halves are added through LDS, the K slices by qgemv_reduce_kernel, both in a fixed order
-// (no float atomics).
+// and handed to the lanes that multiply them through a small LDS slot private to the wave --
+// unless any 16 columns of the group can share an A operand (per-tensor scales, or M <= 4 with
+// the rows packed as below): then lane c loads the 8 columns 8 c .. 8 c + 7 of its own 8 k rows
+// (8 or 4 bytes per row) and multiplies them straight from the registers, MFMA j taking column j
+// of every lane. The two halves are added through LDS, the K slices by qgemv_reduce_kernel,
+// both in a fixed order (no float atomics).
 #include <algorithm>
 #include <type_traits>
 
@@ -93,7 +96,13 @@ __device__ __forceinline__ float quad_lane(uint32_t v) {
 // vector-ALU work: 32 of 60 instructions per 1024 weights). Every block's MFMAs then take the same
 // A operand, and of a block's accumulator only rows 4 u .. 4 u + 3 (the lanes with kg == u) are its
 // product; the others multiply another block's scales and are dropped.
-template <int VPL, bool PER_TENSOR, bool X_BF16, int MT, int SB = 0, bool PK = false>
+// DL (PK or PER_TENSOR): direct loads, no LDS slot. With the slot, the 16 columns of an MFMA must
+// lie in one scale block, which fixes which word a lane needs; here every column of the group
+// meets the same A operand (PK: its block's scales are rows 4 b .. 4 b + 3 of it), so a lane can
+// multiply whatever columns it loaded. Measured on the 4096 x 14336 weight, whole product: Q8S
+// block-32 M = 4 20.9 -> 20.1 us, per-tensor M = 4 / 16 / 32 20.0 / 21.3 / 27.1 -> 18.2 / 20.3 /
+// 26.2 us; Q4S block-32 M = 3 / 4 18.6 / 19.5 -> 17.1 / 17.7 us.
+template <int VPL, bool PER_TENSOR, bool X_BF16, int MT, int SB = 0, bool PK = false, bool DL = false>
 __global__ void __launch_bounds__(kSplitThreads)
 qsplit_kernel(const void* __restrict__ x, const uint32_t* __restrict__ w, const float* __restrict__ scales,
               size_t M, size_t K, size_t N, size_t k_per_wg, float* __restrict__ part) {
@@ -142,8 +151,10 @@ qsplit_kernel(const void* __restrict__ x, const uint32_t* __restrict__ w, const 
   const __amdgpu_buffer_rsrc_t rsrc_s = __builtin_amdgcn_make_buffer_rsrc(
       const_cast<float*>(scales), 0, static_cast<int>(PER_TENSOR ? 4 : K * spr * 4), 0x00020000);
   const uint32_t w_row_bytes = static_cast<uint32_t>(NW * 4), s_row_bytes = static_cast<uint32_t>(spr * 4);
-  const uint32_t w_lane = static_cast<uint32_t>(lane / LPR) * w_row_bytes + static_cast<uint32_t>(gc) * ROW_B +
-                          static_cast<uint32_t>(lane % LPR) * 16u;
+  static_assert(!DL || PK || PER_TENSOR, "direct loads: any 16 columns of the group share their activations");
+  const uint32_t w_lane = DL ? static_cast<uint32_t>(8 * kg) * w_row_bytes + static_cast<uint32_t>(gc) * ROW_B + static_cast<uint32_t>(c) * (ROW_B / 16)
+                             : static_cast<uint32_t>(lane / LPR) * w_row_bytes + static_cast<uint32_t>(gc) * ROW_B +
+                                   static_cast<uint32_t>(lane % LPR) * 16u;
   static_assert(!PK || (MT == 1 && SB == 0 && !PER_TENSOR), "row packing: one tile of rows, one scale per 32 columns");
   // PK: lane (row c % 4, block c / 4) loads that block's scale for k rows 8 kg + c % 4 and + 4
   const uint32_t s_lane = PK ? static_cast<uint32_t>(8 * kg + (c & 3)) * s_row_bytes + static_cast<uint32_t>(gc * 4 + (c >> 2)) * 4u
@@ -175,6 +186,7 @@ qsplit_kernel(const void* __restrict__ x, const uint32_t* __restrict__ w, const 
   // kDepth steps are in flight per wave. Scales: lane (c, kg) loads those of row 8 kg + c % 8 (four
   // blocks, 16 bytes); the multiply reads row r's from lane r of its row of 16 lanes (DPP broadcast).
   vuint4 wl[kDepth][NLOAD];
+  vuint2 wd[kDepth][8];
   vuint4 sq[kDepth];
   // A step past the end of the wave's rows loads nothing: its lane offsets are out of the buffers'
   // range, so the loads return zeros without touching memory. Every fetch and multiply then runs
@@ -185,9 +197,18 @@ qsplit_kernel(const void* __restrict__ x, const uint32_t* __restrict__ w, const 
     const bool ok = s < steps;
     const uint32_t row0 = ok ? static_cast<uint32_t>(kw0) + static_cast<uint32_t>(s) * kStepRows : 0u;
     const uint32_t wo = ok ? w_lane : 0x80000000u, so = ok ? s_lane : 0x80000000u;
+    if (DL) {
 #pragma unroll
-    for (int i = 0; i < NLOAD; ++i)
-      wl[buf][i] = __builtin_amdgcn_raw_buffer_load_b128(rsrc_w, wo, (row0 + static_cast<uint32_t>(RPI * i)) * w_row_bytes, 0);
+      for (int r = 0; r < 8; ++r) {
+        const uint32_t row = (row0 + static_cast<uint32_t>(r)) * w_row_bytes;
+        if (VPL == 4) wd[buf][r] = __builtin_amdgcn_raw_buffer_load_b64(rsrc_w, wo, row, 0);
+        else wd[buf][r] = vuint2{__builtin_amdgcn_raw_buffer_load_b32(rsrc_w, wo, row, 0), 0u};
+      }
+    } else {
+#pragma unroll
+      for (int i = 0; i < NLOAD; ++i)
+        wl[buf][i] = __builtin_amdgcn_raw_buffer_load_b128(rsrc_w, wo, (row0 + static_cast<uint32_t>(RPI * i)) * w_row_bytes, 0);
+    }
     if (PK) {
       sq[buf] = vuint4{__builtin_amdgcn_raw_buffer_load_b32(rsrc_s, so, row0 * s_row_bytes, 0),
                        __builtin_amdgcn_raw_buffer_load_b32(rsrc_s, so, (row0 + 4u) * s_row_bytes, 0), 0u, 0u};
@@ -247,14 +268,17 @@ qsplit_kernel(const void* __restrict__ x, const uint32_t* __restrict__ w, const 
       xv[t][4] = x1.x; xv[t][5] = x1.y; xv[t][6] = x1.z; xv[t][7] = x1.w;
     }
     // through the wave's slot (LDS runs a wave's instructions in order: no barrier)
+    if (!DL) {
 #pragma unroll
-    for (int i = 0; i < NLOAD; ++i) *reinterpret_cast<vuint4*>(slot + slot_wr[i]) = wl[buf][i];
+      for (int i = 0; i < NLOAD; ++i) *reinterpret_cast<vuint4*>(slot + slot_wr[i]) = wl[buf][i];
+    }
     const vuint4 sqv = sq[buf];
     uint32_t wq[kUnits][8];
 #pragma unroll
     for (int u = 0; u < kUnits; ++u)
 #pragma unroll
-      for (int r = 0; r < 8; ++r) wq[u][r] = *reinterpret_cast<const uint32_t*>(slot + slot_rd[u] + ROW_B * r);
+      for (int r = 0; r < 8; ++r)
+        wq[u][r] = DL ? (VPL == 4 && u >> 1 ? wd[buf][r].y : wd[buf][r].x) : *reinterpret_cast<const uint32_t*>(slot + slot_rd[u] + ROW_B * r);
     uint32_t hi[MT][4], lo[MT][4];
     if (PK) {
       const uint32_t a = sqv.x, b = sqv.y;
@@ -292,20 +316,21 @@ qsplit_kernel(const void* __restrict__ x, const uint32_t* __restrict__ w, const 
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
         if (VPL == 4) {
-          const uint32_t p = __builtin_amdgcn_perm(wq[u][2 * i + 1], wq[u][2 * i], sel);
+          // DL: unit u multiplies bytes u % 2 and u % 2 + 2 of word u / 2 of the lane's 8 bytes
+          const uint32_t p = __builtin_amdgcn_perm(wq[u][2 * i + 1], wq[u][2 * i], DL ? (u & 1 ? 0x07030501u : 0x06020400u) : sel);
           b0[i] = __builtin_amdgcn_perm(as_bits(byte_to_float(p, 1)), as_bits(byte_to_float(p, 0)), 0x07060302u);
           b1[i] = __builtin_amdgcn_perm(as_bits(byte_to_float(p, 3)), as_bits(byte_to_float(p, 2)), 0x07060302u);
         } else if (guard) {
           // the nibbles' own values (q = (n ^ 8) - 8, exact in bf16: the upper half of the f32)
-          const uint32_t na = (wq[u][2 * i] >> nib_shift) & 0x000F000Fu, nb = (wq[u][2 * i + 1] >> nib_shift) & 0x000F000Fu;
+          const uint32_t na = (wq[u][2 * i] >> (DL ? 4u * u : nib_shift)) & 0x000F000Fu, nb = (wq[u][2 * i + 1] >> (DL ? 4u * u : nib_shift)) & 0x000F000Fu;
           auto qf = [](uint32_t n) { return as_bits(static_cast<float>(static_cast<int>(n ^ 8u) - 8)); };
           b0[i] = __builtin_amdgcn_perm(qf(nb & 0xFu), qf(na & 0xFu), 0x07060302u);
           b1[i] = __builtin_amdgcn_perm(qf(nb >> 16), qf(na >> 16), 0x07060302u);
         } else {
           // nibble n (two's complement) -> bf16 bits 0x4300 | (n ^ 8) = 128 + (q + 8) = q + 136, both
           // nibbles of the lane at once; the 136 is taken out again by the constant operand below
-          const uint32_t ta = ((wq[u][2 * i] >> nib_shift) & 0x000F000Fu) ^ 0x43084308u;
-          const uint32_t tb = ((wq[u][2 * i + 1] >> nib_shift) & 0x000F000Fu) ^ 0x43084308u;
+          const uint32_t ta = ((wq[u][2 * i] >> (DL ? 4u * u : nib_shift)) & 0x000F000Fu) ^ 0x43084308u;
+          const uint32_t tb = ((wq[u][2 * i + 1] >> (DL ? 4u * u : nib_shift)) & 0x000F000Fu) ^ 0x43084308u;
           b0[i] = __builtin_amdgcn_perm(tb, ta, 0x05040100u);
           b1[i] = __builtin_amdgcn_perm(tb, ta, 0x07060302u);
         }
@@ -428,11 +453,23 @@ qsplit_kernel(const void* __restrict__ x, const uint32_t* __restrict__ w, const 
   __syncthreads();
   float* const stage = reinterpret_cast<float*>(smem);
   constexpr uint32_t SP = kTileCols + 4;  // pitch in floats
-  const uint32_t cell0 = static_cast<uint32_t>(4 * kg) * SP + static_cast<uint32_t>(g) * kGroupCols +
-                         static_cast<uint32_t>(VPL * (c % WPB) + c / WPB);
   // PK: block u's product sits in rows 4 u .. 4 u + 3 of its accumulators, i.e. in the lanes with
-  // kg == u, element i = activation row i.
-  const uint32_t cellp = static_cast<uint32_t>(g) * kGroupCols + static_cast<uint32_t>(VPL * (c % WPB) + c / WPB);
+  // kg == u, element i = activation row i. DL: the lane's columns are 8 c .. 8 c + 7 of the group
+  // (block c / 4), accumulator (u, p) being byte u % 2 + 2 p of word u / 2.
+  auto cell = [&](int t, int u, int p, int i, bool& mine) -> uint32_t {
+    const uint32_t col = static_cast<uint32_t>(g) * kGroupCols;
+    mine = true;
+    if (DL) {
+      mine = !PK || kg == (c >> 2);
+      return (PK ? i : 16 * t + 4 * kg + i) * SP + col + 8u * static_cast<uint32_t>(c) + (VPL == 4 ? 4 * (u >> 1) + (u & 1) + 2 * p : u + 4 * p);
+    }
+    const uint32_t in_block = static_cast<uint32_t>(VPL * (c % WPB) + c / WPB) + 32 * u + (VPL / 2) * p;
+    if (PK) {
+      mine = kg == u;
+      return i * SP + col + in_block;
+    }
+    return (16 * t + 4 * kg + i) * SP + col + in_block;
+  };
   if (h == 1) {
 #pragma unroll
     for (int t = 0; t < MT; ++t)
@@ -442,11 +479,9 @@ qsplit_kernel(const void* __restrict__ x, const uint32_t* __restrict__ w, const 
         for (int p = 0; p < 2; ++p)
 #pragma unroll
           for (int i = 0; i < 4; ++i) {
-            if (PK) {
-              if (kg == u) stage[cellp + i * SP + 32 * u + (VPL / 2) * p] = acc[t][u][p][i];
-            } else {
-              stage[cell0 + (16 * t + i) * SP + 32 * u + (VPL / 2) * p] = acc[t][u][p][i];
-            }
+            bool mine;
+            const uint32_t at = cell(t, u, p, i, mine);
+            if (mine) stage[at] = acc[t][u][p][i];
           }
   }
   __syncthreads();
@@ -459,11 +494,9 @@ qsplit_kernel(const void* __restrict__ x, const uint32_t* __restrict__ w, const 
         for (int p = 0; p < 2; ++p)
 #pragma unroll
           for (int i = 0; i < 4; ++i) {
-            if (PK) {
-              if (kg == u) stage[cellp + i * SP + 32 * u + (VPL / 2) * p] += acc[t][u][p][i];
-            } else {
-              stage[cell0 + (16 * t + i) * SP + 32 * u + (VPL / 2) * p] += acc[t][u][p][i];
-            }
+            bool mine;
+            const uint32_t at = cell(t, u, p, i, mine);
+            if (mine) stage[at] += acc[t][u][p][i];
           }
   }
   __syncthreads();
@@ -523,7 +556,7 @@ bq_status launch_qsplit(const void* x, int x_dtype, const uint32_t* w, const flo
   dim3 grid(p.tiles, p.slices), tb(kSplitThreads);
 #define BQ_SPLIT3(V, PT, XB, T, S, P)                                                              \
   do {                                                                                            \
-    auto kernel = qsplit_kernel<V, PT, XB, T, S, P>;                                              \
+    auto kernel = qsplit_kernel<V, PT, XB, T, S, P, (P || PT)>;                                            \
     /* more than the default 64 KiB: checked against what the device grants, else refused here */ \
     BQ_TRY(configure_dynamic_lds(reinterpret_cast<const void*>(kernel), lds, "qsplit_kernel"));   \
     hipLaunchKernelGGL(kernel, grid, tb, lds, st, x, w, scales, m, k, n, p.k_per_wg, part);       \
