@@ -5,8 +5,9 @@
 // scale per tensor or per run of `block` values along N (scales[k][n / block]). The reference
 // (crates/burn-ndarray/src/ops/qtensor.rs:223-267) materialises dequantize(W) and calls an sgemm;
 // here the dequantize is fused into the operand path:
-//   * decode (f32 lhs: M <= 3 on 8-bit weights, M <= 2 on 4-bit ones; bf16 lhs: M <= 2): a q-GEMV
-//     that unpacks in registers, split over K; HBM bound.
+//   * decode (f32 lhs: M <= 2 on 8-bit weights, M = 1 on 4-bit ones, one row more when the scales
+//     are per 64 or 128 columns; bf16 lhs: M <= 2): a q-GEMV that unpacks in registers, split
+//     over K; HBM bound.
 //   * from there up to M = 32: the split-activation kernel of qsplit.hip (bf16 matrix cores, exact
 //     integer weights, activations x scale as two bf16 terms); the weight layouts it does not take
 //     fall back to the decode kernel (M <= 8), the kernels of qskinny.hip, or the general q-GEMV
@@ -642,10 +643,17 @@ using namespace bq;
 
 static bool use_gemv(size_t m, int32_t lhs_dtype) { return m <= 16 && lhs_dtype == BQ_F32; }
 // Batch size from which the split-activation MFMA kernel beats the vector-ALU decode kernel on
-// the 4096 x 14336 weight. Q8S: decode 16.5 / 18.7 / 20.3 / 22.6 us for M = 1..4, the matrix-core
-// kernel 21 us for M = 3 and 4 (its row-packed form, M <= 4) and 22-24.5 us above. Q4S: decode
-// 14.6 / 17.0 us for M = 1, 2, the matrix-core kernel 17.9 us for M = 3 and 4.
-static size_t split_from_m(int value) { return value == BQ_Q8S ? 4 : 3; }
+// the 4096 x 14336 weight, one run (us per product, decode / matrix-core kernel). With the weights
+// loaded directly (per-tensor scales or one scale per 32 columns), Q8S per tensor: M = 2 17.1 /
+// 17.4, M = 3 18.6 / 17.3, M = 4 21.5 / 17.5; Q8S block-32: 19.5 / 19.8, 21.1 / 19.8, 23.5 / 19.9;
+// Q4S per tensor: 16.0 / 15.9, 18.5 / 15.7, 20.7 / 15.7; Q4S block-32: 18.1 / 16.5, 22.1 / 16.5,
+// 22.9 / 16.5. Through the LDS slot (one scale per 64 or 128 columns) the matrix-core kernel
+// takes 22-24.5 us, and the decode kernel stays ahead one row longer.
+static size_t split_from_m(int value, int block) {
+  const bool direct = block == 0 || block == 32;
+  if (value == BQ_Q8S) return direct ? 3 : 4;
+  return direct ? 2 : 3;
+}
 
 namespace bq {
 // Whether bqk_q_matmul has a fused kernel for this problem (else: dequantize + float matmul).
@@ -751,7 +759,7 @@ static bq_status q_matmul_core(const void* lhs, int32_t lhs_dtype, size_t m, siz
   const bool bf16_decode = lhs_dtype == BQ_BF16 && gemv1_ok(m, n, lhs_dtype, block, value) &&
                            (reinterpret_cast<uintptr_t>(w_values) & 15u) == 0 && (reinterpret_cast<uintptr_t>(lhs) & 3u) == 0 &&
                            k % 2 == 0;  // (whole 32-bit words of activations)
-  if ((m >= split_from_m(value) || (lhs_dtype == BQ_BF16 && !bf16_decode)) && split_ok(m, k, n, lhs_dtype, value, block) &&
+  if ((m >= split_from_m(value, block) || (lhs_dtype == BQ_BF16 && !bf16_decode)) && split_ok(m, k, n, lhs_dtype, value, block) &&
       (reinterpret_cast<uintptr_t>(w_values) & 15u) == 0 &&
       (per_tensor || (reinterpret_cast<uintptr_t>(w_scales) & 15u) == 0)) {
     const size_t need = split_workspace(m, k, n);

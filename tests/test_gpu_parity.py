@@ -1573,9 +1573,11 @@ def test_q_matmul_split_k_tiles(dev, value, block, m, k, n):
 @pytest.mark.parametrize("block", [None, (32,), (64,)])
 @pytest.mark.parametrize("m,k,n", [(1, 4096, 1024), (2, 1000, 448), (1, 130, 64), (2, 64, 4096)])
 def test_bf16_decode_is_the_f32_decode_on_widened_activations(dev, value, block, m, k, n):
-    """One or two rows of bf16 activations take the decode kernel, which widens them exactly:
-    the same bits as the f32 activations of the same values, and within f32 rounding of the
-    float64 product."""
+    """One or two rows of bf16 activations take the kernel f32 activations take and are widened
+    exactly: the same bits as for the f32 activations of the same values. The decode kernel is
+    within f32 rounding of the float64 product; two rows over 4-bit weights whose scales are per
+    tensor or per 32 columns take the split-activation kernel where its layout applies (16
+    significant bits per product)."""
     rng = np.random.default_rng(m * 17 + k + n)
     w = (rng.standard_normal((k, n)) * 0.05).astype(np.float32)
     xb = ba.bf16_bits_from_f32(rng.standard_normal((m, k)).astype(np.float32))
@@ -1588,7 +1590,8 @@ def test_bf16_decode_is_the_f32_decode_on_widened_activations(dev, value, block,
         QTensorOps.q_matmul(FloatOps.float_from_data(xb, dev, ba.BF16), tq, out_dtype=ba.F32))
     out_f = FloatOps.float_into_data(QTensorOps.q_matmul(FloatOps.float_from_data(x, dev), tq))
     assert out_b.tobytes() == out_f.tobytes()
-    assert np.abs(out_b - ref).max() <= 2e-6 * np.abs(ref).max()
+    split = m == 2 and value == QuantValue.Q4S and block in (None, (32,)) and n % 128 == 0 and k % 32 == 0
+    assert np.abs(out_b - ref).max() <= (2e-5 if split else 2e-6) * np.abs(ref).max()
     # default output dtype follows the activations
     out_h = QTensorOps.q_matmul(FloatOps.float_from_data(xb, dev, ba.BF16), tq)
     assert out_h.dtype == ba.BF16
