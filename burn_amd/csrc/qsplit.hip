@@ -21,9 +21,14 @@
 // Q8S: the per-lane field choice is made by v_perm_b32 with a per-lane selector, which gathers
 // the two fields of two rows into one register; sign-extending byte converts (SDWA) and a second
 // v_perm_b32 (the upper halves of two floats are their bf16) finish the operand. Q4S: a per-lane
-// shift brings the lane's two nibbles to the low nibble of each 16-bit half, and and + xor turn
-// them into the bf16 bit patterns of q + 136 (0x4300 | (nibble ^ 8)); the 136 comes off again in
-// the same accumulators through two more MFMAs against a constant -136 operand.
+// rotation brings the lane's two nibbles to bits 3..6 of each 16-bit half, and and + xor turn
+// them into the bf16 bit patterns 0x4180 | (nibble ^ 8) << 3 = 16 + (q + 8) = q + 24 (the nibble
+// in the upper 4 of the 7 mantissa bits: exact); the 24 comes off through two more MFMAs per
+// distinct A operand against a constant -24 operand, into an accumulator of their own that is
+// added when the tile is stored (every column of it holds 24 times the sum of the row's
+// activations). With the 0x4300 | (nibble ^ 8) = q + 136 patterns and the correction taken in
+// every accumulator, the same kernels measured 1-4 us more and an error of 3.5e-6 to 7e-6 of
+// the largest output instead of 2.9e-6 to 4.9e-6.
 //
 // A wave owns 4 adjacent blocks (128 columns: a row is 128 bytes of Q8S or 64 of Q4S) and a run
 // of k rows; the 8 waves of a workgroup are 4 such column groups x 2 halves of the workgroup's K
@@ -172,16 +177,25 @@ qsplit_kernel(const void* __restrict__ x, const uint32_t* __restrict__ w, const 
   const float s_tensor = PER_TENSOR ? scales[0] : 0.0f;
   // Q8S: v_perm_b32 selector: bytes (f0 of row a, f0 of row b, f0 + 2 of row a, f0 + 2 of row b).
   // Q4S: the lane's two nibbles f0 and f0 + 4 of a word are 16 bits apart: one shift by 4 f0
-  // brings them to the low nibble of each half.
+  // brings them to the low nibble of each half (guarded loop), one rotation to bits 3..6.
   const uint32_t f0 = static_cast<uint32_t>(c / WPB);
   const uint32_t sel = f0 | ((4u + f0) << 8) | ((f0 + 2u) << 16) | ((6u + f0) << 24);
   const uint32_t nib_shift = 4u * f0;
+  const uint32_t nib_rot = (4u * f0 + 29u) & 31u;  // rotate right: nibble f0 to bits 3..6, nibble f0 + 4 to bits 19..22
 
   floatx4 acc[MT][kUnits][2];
+  // Q4S: the offset of the weight patterns times the sum of the activations, one accumulator per
+  // distinct A operand (every column of it holds the same value)
+  constexpr bool kSharedA = PK || PER_TENSOR;  // the wave's 4 units multiply the same A operand
+  constexpr int kOffsetAccs = kSharedA ? 1 : kUnits;
+  floatx4 off[MT][kOffsetAccs];
 #pragma unroll
-  for (int t = 0; t < MT; ++t)
+  for (int t = 0; t < MT; ++t) {
 #pragma unroll
     for (int u = 0; u < kUnits; ++u) acc[t][u][0] = acc[t][u][1] = floatx4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int u = 0; u < kOffsetAccs; ++u) off[t][u] = floatx4{0.f, 0.f, 0.f, 0.f};
+  }
 
   // kDepth steps are in flight per wave. Scales: lane (c, kg) loads those of row 8 kg + c % 8 (four
   // blocks, 16 bytes); the multiply reads row r's from lane r of its row of 16 lanes (DPP broadcast).
@@ -227,7 +241,7 @@ qsplit_kernel(const void* __restrict__ x, const uint32_t* __restrict__ w, const 
   // holds an infinity or a NaN. There the second term of a non-finite product is dropped (inf - inf
   // would make every output of the row NaN, where the reference's sum has +-inf, and NaN only
   // against a zero weight), Q4S weights are converted to their true values instead of the offset
-  // patterns (inf * (q + 136) - inf * 136 is NaN), and the padded step past the end is skipped
+  // patterns (inf * (q + 24) - inf * 24 is NaN), and the padded step past the end is skipped
   // (inf * 0). Finite slices never execute any of it.
   // (-1, 0) and (0, -1) as bf16 pairs, kept in registers the compiler cannot see through: written
   // as constants, (-1, 0) becomes the inline operand -1.0, which this instruction reads as the 32-bit
@@ -298,6 +312,36 @@ qsplit_kernel(const void* __restrict__ x, const uint32_t* __restrict__ w, const 
         split(G, v, hi[t], lo[t]);
       }
     }
+    // Q4S with direct loads: the lane's word of a row holds its 8 columns, one nibble each, and all
+    // 4 units read the same words. Two byte permutes gather bytes 0, 2 (nibbles 0, 1, 4, 5) and
+    // bytes 1, 3 (nibbles 2, 3, 6, 7) of two rows; after one xor (n ^ 8 in every nibble) a shift and
+    // an and-or leave, per unit, the 4 bytes 0x80 | (n ^ 8) << 3 of (row a, row b) x (nibble u,
+    // nibble u + 4): the low bytes of the bf16 patterns 0x4180 | (n ^ 8) << 3 = 16 + (q + 8) = q + 24.
+    uint32_t nlo[4][kUnits];
+    if (VPL == 8 && DL && !guard) {
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const uint32_t wa = wd[buf][2 * i].x, wb = wd[buf][2 * i + 1].x;
+        const uint32_t p01 = __builtin_amdgcn_perm(wb, wa, 0x06020400u) ^ 0x88888888u;
+        const uint32_t p23 = __builtin_amdgcn_perm(wb, wa, 0x07030501u) ^ 0x88888888u;
+        nlo[i][0] = ((p01 << 3) & 0x78787878u) | 0x80808080u;
+        nlo[i][1] = ((p01 >> 1) & 0x78787878u) | 0x80808080u;
+        nlo[i][2] = ((p23 << 3) & 0x78787878u) | 0x80808080u;
+        nlo[i][3] = ((p23 >> 1) & 0x78787878u) | 0x80808080u;
+      }
+    }
+    // the offset comes off through two MFMAs per distinct A operand against a constant -24
+    const bf16x8 minus = __builtin_bit_cast(bf16x8, vuint4{0xC1C0C1C0u, 0xC1C0C1C0u, 0xC1C0C1C0u, 0xC1C0C1C0u});
+    auto take_offset = [&](int u) {
+#pragma unroll
+      for (int t = 0; t < MT; ++t) {
+        const bf16x8 a_hi = __builtin_bit_cast(bf16x8, vuint4{hi[t][0], hi[t][1], hi[t][2], hi[t][3]});
+        const bf16x8 a_lo = __builtin_bit_cast(bf16x8, vuint4{lo[t][0], lo[t][1], lo[t][2], lo[t][3]});
+        off[t][u] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a_hi, minus, off[t][u], 0, 0, 0);
+        off[t][u] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a_lo, minus, off[t][u], 0, 0, 0);
+      }
+    };
+    if (VPL == 8 && !guard && kSharedA) take_offset(0);
 #pragma unroll
     for (int u = 0; u < kUnits; ++u) {
       if (!PER_TENSOR && !PK) {
@@ -311,6 +355,7 @@ qsplit_kernel(const void* __restrict__ x, const uint32_t* __restrict__ w, const 
           for (int r = 0; r < 8; ++r) v[r] = xv[t][r] * sr[r];
           split(G, v, hi[t], lo[t]);
         }
+        if (VPL == 8 && !guard) take_offset(u);
       }
       uint32_t b0[4], b1[4];
 #pragma unroll
@@ -326,35 +371,31 @@ qsplit_kernel(const void* __restrict__ x, const uint32_t* __restrict__ w, const 
           auto qf = [](uint32_t n) { return as_bits(static_cast<float>(static_cast<int>(n ^ 8u) - 8)); };
           b0[i] = __builtin_amdgcn_perm(qf(nb & 0xFu), qf(na & 0xFu), 0x07060302u);
           b1[i] = __builtin_amdgcn_perm(qf(nb >> 16), qf(na >> 16), 0x07060302u);
+        } else if (DL) {
+          // low bytes from above under the constant high byte 0x41: (row a, row b) of nibble u, of nibble u + 4
+          b0[i] = __builtin_amdgcn_perm(0x41414141u, nlo[i][u], 0x04010400u);
+          b1[i] = __builtin_amdgcn_perm(0x41414141u, nlo[i][u], 0x04030402u);
         } else {
-          // nibble n (two's complement) -> bf16 bits 0x4300 | (n ^ 8) = 128 + (q + 8) = q + 136, both
-          // nibbles of the lane at once; the 136 is taken out again by the constant operand below
-          const uint32_t ta = ((wq[u][2 * i] >> (DL ? 4u * u : nib_shift)) & 0x000F000Fu) ^ 0x43084308u;
-          const uint32_t tb = ((wq[u][2 * i + 1] >> (DL ? 4u * u : nib_shift)) & 0x000F000Fu) ^ 0x43084308u;
+          // the same pattern from the lane's own word of the unit: a rotation brings its nibbles f0
+          // and f0 + 4 (16 bits apart) to bits 3..6 of each half, and and + xor finish both at once.
+          // (Gathering the bytes of two rows first, as above, saves two instructions per pair here
+          // too and was not faster: 22.3 against 21.8 us at M = 16.)
+          const uint32_t ta = (__builtin_amdgcn_alignbit(wq[u][2 * i], wq[u][2 * i], nib_rot) & 0x00780078u) ^ 0x41C041C0u;
+          const uint32_t tb = (__builtin_amdgcn_alignbit(wq[u][2 * i + 1], wq[u][2 * i + 1], nib_rot) & 0x00780078u) ^ 0x41C041C0u;
           b0[i] = __builtin_amdgcn_perm(tb, ta, 0x05040100u);
           b1[i] = __builtin_amdgcn_perm(tb, ta, 0x07060302u);
         }
       }
       const bf16x8 bq0 = __builtin_bit_cast(bf16x8, vuint4{b0[0], b0[1], b0[2], b0[3]});
       const bf16x8 bq1 = __builtin_bit_cast(bf16x8, vuint4{b1[0], b1[1], b1[2], b1[3]});
-      // (q + 136) - 136 for Q4S: every column times bf16(-136) = 0xC308
-      const bf16x8 minus = __builtin_bit_cast(bf16x8, vuint4{0xC308C308u, 0xC308C308u, 0xC308C308u, 0xC308C308u});
 #pragma unroll
       for (int t = 0; t < MT; ++t) {
         const bf16x8 a_hi = __builtin_bit_cast(bf16x8, vuint4{hi[t][0], hi[t][1], hi[t][2], hi[t][3]});
         const bf16x8 a_lo = __builtin_bit_cast(bf16x8, vuint4{lo[t][0], lo[t][1], lo[t][2], lo[t][3]});
         acc[t][u][0] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a_hi, bq0, acc[t][u][0], 0, 0, 0);
         acc[t][u][1] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a_hi, bq1, acc[t][u][1], 0, 0, 0);
-        if (VPL == 8 && !guard) {
-          acc[t][u][0] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a_hi, minus, acc[t][u][0], 0, 0, 0);
-          acc[t][u][1] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a_hi, minus, acc[t][u][1], 0, 0, 0);
-        }
         acc[t][u][0] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a_lo, bq0, acc[t][u][0], 0, 0, 0);
         acc[t][u][1] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a_lo, bq1, acc[t][u][1], 0, 0, 0);
-        if (VPL == 8 && !guard) {
-          acc[t][u][0] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a_lo, minus, acc[t][u][0], 0, 0, 0);
-          acc[t][u][1] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a_lo, minus, acc[t][u][1], 0, 0, 0);
-        }
       }
     }
   };
@@ -481,7 +522,7 @@ qsplit_kernel(const void* __restrict__ x, const uint32_t* __restrict__ w, const 
           for (int i = 0; i < 4; ++i) {
             bool mine;
             const uint32_t at = cell(t, u, p, i, mine);
-            if (mine) stage[at] = acc[t][u][p][i];
+            if (mine) stage[at] = acc[t][u][p][i] + (VPL == 8 ? off[t][kSharedA ? 0 : u][i] : 0.0f);
           }
   }
   __syncthreads();
@@ -496,7 +537,7 @@ qsplit_kernel(const void* __restrict__ x, const uint32_t* __restrict__ w, const 
           for (int i = 0; i < 4; ++i) {
             bool mine;
             const uint32_t at = cell(t, u, p, i, mine);
-            if (mine) stage[at] += acc[t][u][p][i];
+            if (mine) stage[at] += acc[t][u][p][i] + (VPL == 8 ? off[t][kSharedA ? 0 : u][i] : 0.0f);
           }
   }
   __syncthreads();
