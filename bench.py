@@ -513,6 +513,27 @@ def run_next(ba, dev, steps, warmup, cpu):
     del ws, w0, blob, values, scales
     dev.trim()
 
+    # ---- the same products over a 4-bit weight ------------------------------------------------------
+    w0 = quantized_weight(ba, dev, 0xC4, (k, n), QuantValue.Q4S)
+    blob = QTensorOps.q_into_data(w0)
+    ws = [w0] + [QTensorOps.q_from_data(blob, dev) for _ in range(15)]
+    values, scales = blob.split()
+    wd = unpack_columns(values, scales, k, n, cols, q4=True)
+    q4 = {}
+    for m in (1, 4, 16):
+        xh = rng.standard_normal((m, k), dtype=np.float32)
+        x = FloatOps.float_from_data(xh, dev)
+        got = FloatOps.float_into_data(QTensorOps.q_matmul(x, ws[5]))[:, cols]
+        rel = matmul_gate(f"Q4S M={m}", got, xh.astype(np.float64) @ wd)
+        t_mm = graph_ms(dev, lambda: [QTensorOps.q_matmul(x, wq) for wq in ws], 16, steps, warmup)
+        wb = k * n // 2 + 4 * k * n // 32
+        q4[f"M={m}"] = {"ms": t_mm, "weight_GB/s": wb / t_mm / 1e6, "frac_hbm": wb / t_mm / 1e6 / HBM_PEAK_GBS,
+                        "max_normalised_error": rel}
+    out["q4s_small_batch"] = {"workload": "x[M,4096] f32 x Q4S block-32 PackedU32 [4096,14336] -> f32 (C4's shape, half the weight bytes)",
+                              "parity": "vs float64 on every 37th column, rel 1e-2 and burn's elementwise rule", **q4}
+    del ws, w0, blob, values, scales
+    dev.trim()
+
     # ---- scale dtypes: quantize_dynamic + dequantize of C2's tensor ------------------------------
     rows = 8192
     nel = rows * 8192
