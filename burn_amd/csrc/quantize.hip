@@ -148,17 +148,21 @@ __device__ __forceinline__ void store_words_quad(uint32_t (&packed)[4], size_t c
   else *reinterpret_cast<vuint4*>(out + at) = v;
 }
 
-// ---- the second of two passes runs back to front -------------------------------------------------
+// ---- the second of two passes goes to the XCD that read each chunk in the first -------------------
 // A per-tensor scale (alone, or over block scales) needs max|x| of the whole tensor before a value
 // can be quantized: absmax_kernel reads the tensor front to back, in chunks of kThreads *
-// kAbsmaxUnroll float4s, and what it read last is still in the L2 of the XCD that read it --
-// workgroups go to the 8 XCDs round robin, so chunk c sits in XCD c % 8. The pass that quantizes
-// takes pieces of PPC to the chunk, back to front, and workgroup b, which lands on XCD b % 8,
-// takes a piece of a chunk that XCD read: on a 4096 x 4096 tensor the per-tensor second pass
-// takes 12.4 us instead of 14.4 (both passes 24.8 instead of 27.1). `grid` is a multiple of
-// 8 * PPC; pieces past the end of the tensor find nothing to do. (Streaming loads in the first
-// pass for all but the last 16-32 MB, to keep exactly those: 25.3-26.2 us. 1024 or 2048
-// first-pass workgroups instead of 512: 25.8-26.7 us.)
+// kAbsmaxUnroll float4s. Workgroups go to the 8 XCDs round robin, so chunk c was read by XCD
+// c % 8. The pass that quantizes takes pieces of PPC to the chunk, and workgroup b, which lands
+// on XCD b % 8, takes a piece of a chunk that XCD read, starting with the last ones. Measured on
+// a 4096 x 4096 tensor, both passes, one run: 27.0 us with workgroup b on piece b, 26.8 us
+// with the pieces merely reversed, 25.1 us on the first pass's XCD front to back, 24.7 us on
+// the first pass's XCD back to front (the second pass by the profiler: 14.4 -> 12.4 us; alone on
+// a cold tensor it takes 16.8 us under every mapping). What carries over is state of the XCD
+// other than cached data: the L2 hit and miss counts and the bytes requested from the fabric are
+// the same under all four mappings (every line of the input misses again). `grid` is a multiple
+// of 8 * PPC; pieces past the end of the tensor find nothing to do. (Streaming loads in the
+// first pass for all but the last 16-32 MB: 25.3-26.2 us. 1024 or 2048 first-pass workgroups
+// instead of 512: 25.8-26.7 us.)
 constexpr int kAbsmaxUnroll = BQ_ABSMAX_UNROLL;
 template <unsigned PPC>
 __device__ __forceinline__ size_t piece_back_to_front(unsigned b, unsigned grid) {
