@@ -98,9 +98,10 @@ __device__ __forceinline__ float quad_lane(uint32_t v) {
 // PK (M <= 4, one scale per 32 columns): the 16 rows of the A operand are 4 activation rows x the
 // wave's 4 blocks of 32 columns -- lane c prepares row c % 4 against the scales of block c / 4 -- so
 // the split activations are computed once per step instead of once per block (they are most of the
-// vector-ALU work: 32 of 60 instructions per 1024 weights). Every block's MFMAs then take the same
-// A operand, and of a block's accumulator only rows 4 u .. 4 u + 3 (the lanes with kg == u) are its
-// product; the others multiply another block's scales and are dropped.
+// vector-ALU work: 32 of 60 instructions per 1024 weights). Every MFMA of the wave then takes the
+// same A operand, and of a column's 16 accumulator rows only the 4 of its own block b (rows 4 b ..
+// 4 b + 3, held by the lanes with kg == b) are its product; the others multiply another block's
+// scales and are dropped.
 // DL (PK or PER_TENSOR): direct loads, no LDS slot. With the slot, the 16 columns of an MFMA must
 // lie in one scale block, which fixes which word a lane needs; here every column of the group
 // meets the same A operand (PK: its block's scales are rows 4 b .. 4 b + 3 of it), so a lane can
@@ -156,7 +157,7 @@ qsplit_kernel(const void* __restrict__ x, const uint32_t* __restrict__ w, const 
   const __amdgpu_buffer_rsrc_t rsrc_s = __builtin_amdgcn_make_buffer_rsrc(
       const_cast<float*>(scales), 0, static_cast<int>(PER_TENSOR ? 4 : K * spr * 4), 0x00020000);
   const uint32_t w_row_bytes = static_cast<uint32_t>(NW * 4), s_row_bytes = static_cast<uint32_t>(spr * 4);
-  static_assert(!DL || PK || PER_TENSOR, "direct loads: any 16 columns of the group share their activations");
+  static_assert(DL == (PK || PER_TENSOR), "direct loads exactly where any 16 columns of the group share their activations");
   const uint32_t w_lane = DL ? static_cast<uint32_t>(8 * kg) * w_row_bytes + static_cast<uint32_t>(gc) * ROW_B + static_cast<uint32_t>(c) * (ROW_B / 16)
                              : static_cast<uint32_t>(lane / LPR) * w_row_bytes + static_cast<uint32_t>(gc) * ROW_B +
                                    static_cast<uint32_t>(lane % LPR) * 16u;
@@ -494,9 +495,9 @@ qsplit_kernel(const void* __restrict__ x, const uint32_t* __restrict__ w, const 
   __syncthreads();
   float* const stage = reinterpret_cast<float*>(smem);
   constexpr uint32_t SP = kTileCols + 4;  // pitch in floats
-  // PK: block u's product sits in rows 4 u .. 4 u + 3 of its accumulators, i.e. in the lanes with
-  // kg == u, element i = activation row i. DL: the lane's columns are 8 c .. 8 c + 7 of the group
-  // (block c / 4), accumulator (u, p) being byte u % 2 + 2 p of word u / 2.
+  // DL: the lane's columns are 8 c .. 8 c + 7 of the group (block c / 4), accumulator (u, p) being
+  // byte u % 2 + 2 p of word u / 2 (Q4S: nibble u + 4 p). PK: a block's product sits in rows 4 b ..
+  // 4 b + 3 of the accumulators, i.e. in the lanes with kg == b, element i = activation row i.
   auto cell = [&](int t, int u, int p, int i, bool& mine) -> uint32_t {
     const uint32_t col = static_cast<uint32_t>(g) * kGroupCols;
     mine = true;
@@ -505,10 +506,6 @@ qsplit_kernel(const void* __restrict__ x, const uint32_t* __restrict__ w, const 
       return (PK ? i : 16 * t + 4 * kg + i) * SP + col + 8u * static_cast<uint32_t>(c) + (VPL == 4 ? 4 * (u >> 1) + (u & 1) + 2 * p : u + 4 * p);
     }
     const uint32_t in_block = static_cast<uint32_t>(VPL * (c % WPB) + c / WPB) + 32 * u + (VPL / 2) * p;
-    if (PK) {
-      mine = kg == u;
-      return i * SP + col + in_block;
-    }
     return (16 * t + 4 * kg + i) * SP + col + in_block;
   };
   if (h == 1) {
