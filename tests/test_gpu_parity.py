@@ -1494,6 +1494,37 @@ def test_q_matmul_small_batches(dev, value, block, m, k, n):
     assert again.tobytes() == out.tobytes()
 
 
+def test_small_batch_kernels_random_shapes(dev):
+    """200 seeded products with 1 <= M <= 32 over weights in whole 128-column groups and 32-row
+    steps (any number of either, so the last tile and the last K slice are partly empty more often
+    than not): the decode kernel and every form of the split-activation kernel -- row-packed,
+    per-tensor, one scale per 32, 64 or 128 columns, one or two tiles of rows, both value widths,
+    both activation dtypes, activations from 1e-3 to 1e3. Each within 2e-5 of the float64 product
+    of the dequantized weights (the kernels keep 16 significant bits per product or better)."""
+    rng = np.random.default_rng(4242)
+    for case in range(200):
+        value = [QuantValue.Q8S, QuantValue.Q4S, QuantValue.Q8F, QuantValue.Q4F][rng.integers(4)]
+        block = [None, (32,), (64,), (128,)][rng.integers(4)]
+        n, k, m = 128 * int(rng.integers(1, 30)), 32 * int(rng.integers(1, 70)), int(rng.integers(1, 33))
+        w = (rng.standard_normal((k, n)) * 0.05).astype(np.float32)
+        if rng.integers(4) == 0:
+            w[rng.random(w.shape) < 0.5] = 0.0
+        tw = QTensorOps.quantize_dynamic(FloatOps.float_from_data(w, dev), QuantScheme(value=value, block=block))
+        wd = FloatOps.float_into_data(QTensorOps.dequantize(tw)).astype(np.float64)
+        xh = (rng.standard_normal((m, k)) * 10.0 ** rng.integers(-3, 4)).astype(np.float32)
+        bf16 = bool(rng.integers(2))
+        if bf16:
+            bits = ba.bf16_bits_from_f32(xh)
+            xh = ba.f32_from_bf16_bits(bits).reshape(m, k)
+            lhs = FloatOps.float_from_data(bits, dev, ba.BF16)
+        else:
+            lhs = FloatOps.float_from_data(xh, dev)
+        ref = xh.astype(np.float64) @ wd
+        out = FloatOps.float_into_data(QTensorOps.q_matmul(lhs, tw, out_dtype=ba.F32))
+        rel = np.abs(out - ref).max() / max(np.abs(ref).max(), 1e-30)
+        assert rel <= 2e-5, f"case {case}: m={m} k={k} n={n} {value.name} block={block} bf16={bf16}: {rel:.3e}"
+
+
 @pytest.mark.parametrize("value", [QuantValue.Q8S, QuantValue.Q4S])
 @pytest.mark.parametrize("block", [None, (32,), (64,)])
 @pytest.mark.parametrize("m,k,n", [(1, 4096, 1024), (1, 100, 64), (2, 96, 256), (4, 1056, 640), (8, 96, 128),
