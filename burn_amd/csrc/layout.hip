@@ -83,7 +83,18 @@ q8_transpose_kernel(const uint32_t* __restrict__ src, uint32_t* __restrict__ dst
   const size_t plane = static_cast<size_t>(R) * C / 4;  // words per batch entry
   src += plane * blockIdx.z;
   dst += plane * blockIdx.z;
-  const uint32_t r0 = blockIdx.y * kTile, c0 = blockIdx.x * kTile;
+  // Workgroups go to the 8 XCDs round robin. When the tile count allows, each XCD takes a run of
+  // consecutive tiles down a tile column, whose outputs are adjacent 128-byte pieces of the same
+  // output rows, instead of every eighth tile of a tile row ([8192,8192]: 31.6 -> 29.2 us; runs
+  // along a tile row, which share source rows instead: 30.8 us).
+  uint32_t bx = blockIdx.x, by = blockIdx.y;
+  const uint32_t total = gridDim.x * gridDim.y;
+  if (total % 8 == 0) {
+    const uint32_t lin = blockIdx.y * gridDim.x + blockIdx.x, t = (lin & 7u) * (total / 8) + (lin >> 3);
+    by = t % gridDim.y;
+    bx = t / gridDim.y;
+  }
+  const uint32_t r0 = by * kTile, c0 = bx * kTile;
   const uint32_t cw = C / 4, rw = R / 4;
   const uint32_t w = threadIdx.x % kTileWords, q0 = threadIdx.x / kTileWords;  // word column; first row quad (of 8 per pass)
 #pragma unroll
