@@ -220,6 +220,36 @@ def test_reference_transposed_and_permuted_cases(dev, approx):
     approx(np.transpose(roundtrip(np.ascontiguousarray(np.transpose(x, (1, 2, 0, 3))), per_tensor), (2, 0, 1, 3)), x, 1e-2, 1e-1)
 
 
+def test_reference_gpu_backend_quantize_dequantize_cases(dev):
+    """crates/burn-backend-tests/tests/cubecl/quantization/quantize_dequantize.rs, case by case: the
+    reference's GPU backend is checked there against its CPU backend with the Native store; here
+    the same inputs go against the oracle, bit for bit (values, scales, blob, dequantized floats).
+    :112-143 arange [8,16] per tensor, all six values, packed; :145-164 the literal [2,16] tensor
+    in blocks of 8 (Q8S, Q4S, Q2S) and 16 (Q2S); :166-178 Native store; :180-223 arange [32,32] and [128,256] in blocks of 32,
+    both stores; :225-235 a last dim that does not fill packed words is refused."""
+    def arange(shape):
+        return np.arange(int(np.prod(shape)), dtype=np.float32).reshape(shape)
+
+    packed, native = QuantStore.PackedU32, QuantStore.Native
+    for value in (QuantValue.Q8S, QuantValue.Q8F, QuantValue.Q4S, QuantValue.Q4F, QuantValue.Q2S, QuantValue.Q2F):
+        check_quantize_dynamic(dev, arange((8, 16)), QuantScheme(value=value, store=packed))
+    literal = np.float32([[-1.8, -1.0, 0.0, 0.5, -1.8, -1.0, 0.0, 0.5, 0.01, 0.025, 0.03, 0.04, 0.01, 0.025, 0.03, 0.04],
+                          [1.8, 1.0, 0.0, -0.5, 1.8, 1.0, 0.0, -0.5, -0.01, -0.025, -0.03, -0.04, -0.01, -0.025, -0.03, -0.04]])
+    check_quantize_dynamic(dev, literal, QuantScheme(value=QuantValue.Q8S, store=packed).per_block((8,)))
+    check_quantize_dynamic(dev, literal, QuantScheme(value=QuantValue.Q4S, store=packed).per_block((8,)))
+    # should_panic_when_block_size_cannot_store_num_quants: the reference's GPU backend refuses blocks
+    # of 8 two-bit values (half a packed word); its CPU backend takes them, and so does this library
+    check_quantize_dynamic(dev, literal, QuantScheme(value=QuantValue.Q2S, store=packed).per_block((8,)))
+    check_quantize_dynamic(dev, literal, QuantScheme(value=QuantValue.Q2S, store=packed).per_block((16,)))
+    check_quantize_dynamic(dev, arange((32, 32)), QuantScheme(value=QuantValue.Q8S, store=native))
+    check_quantize_dynamic(dev, literal, QuantScheme(value=QuantValue.Q8S, store=native).per_block((8,)))
+    for shape in ((32, 32), (128, 256)):
+        for store in (packed, native):
+            check_quantize_dynamic(dev, arange(shape), QuantScheme(value=QuantValue.Q8S, store=store).per_block((32,)))
+    with pytest.raises(ba.BurnqError):   # should_panic_when_shape_cannot_store_quants: "Can't store in u32"
+        gpu_quantize_dynamic(dev, np.float32([[1.0, 6.35], [2.0, 3.0], [1.0, 3.0]]), QuantScheme(store=packed))
+
+
 # ------------------------------------------------------------------ seeded parity, all schemes
 
 @pytest.mark.parametrize("value", [QuantValue.Q8S, QuantValue.Q4S])
@@ -535,6 +565,41 @@ def test_q_reshape_is_metadata_only(dev):
         QTensorOps.q_reshape(tb, (2, 512))   # one extent of 256
     same = QTensorOps.q_to_device(tq, dev)
     assert QTensorOps.q_into_data(same).bytes.tobytes() == QTensorOps.q_into_data(tq).bytes.tobytes()
+
+
+def test_reference_gpu_backend_reshape_cases(dev, approx):
+    """crates/burn-backend-tests/tests/cubecl/quantization/reshape.rs, case by case: arange / n,
+    quantize_dynamic, reshape, dequantize, against the reshaped input within the permissive
+    tolerance as there, and -- sharper -- bit-equal to dequantize-then-reshape (:157-192). Where the
+    reference's GPU backend refuses a reshape that its CPU backend performs (sub-byte values,
+    :60-82; a block of 32 folded into rows of 16, :127-155) this library performs it like the CPU
+    backend, since the memory order of values and scales does not change; a 2-D block that the new
+    shape cuts is refused by both (:113-125)."""
+    def case(block, value, store, shape, new_shape):
+        n = int(np.prod(shape))
+        x = (np.arange(n, dtype=np.float32) / np.float32(n)).reshape(shape)
+        scheme = QuantScheme(value=value, store=store)
+        if block is not None:
+            scheme = scheme.per_block(block)
+        tq = QTensorOps.quantize_dynamic(FloatOps.float_from_data(x, dev), scheme)
+        d_flat = FloatOps.float_into_data(QTensorOps.dequantize(tq))
+        r = QTensorOps.q_reshape(tq, new_shape)
+        d = FloatOps.float_into_data(QTensorOps.dequantize(r))
+        assert d.shape == tuple(new_shape) and d.tobytes() == d_flat.reshape(new_shape).tobytes()
+        if value == QuantValue.Q8S:   # (the 4-bit cases never reach this comparison in the reference)
+            approx(d, x.reshape(new_shape), 1e-2, 1e-2)
+
+    packed, native = QuantStore.PackedU32, QuantStore.Native
+    case((16,), QuantValue.Q8S, packed, (32,), (2, 16))
+    case((16,), QuantValue.Q4S, packed, (32,), (2, 16))
+    case(None, QuantValue.Q4S, packed, (32,), (2, 16))
+    case((16,), QuantValue.Q8S, native, (32,), (2, 16))
+    case((32,), QuantValue.Q8S, packed, (32,), (1, 1, 1, 32))
+    with pytest.raises(ba.BurnqError):   # quantize_2d_block_reshape_should_panic
+        case((2, 4), QuantValue.Q8S, packed, (4, 8), (32,))
+    case((32,), QuantValue.Q8S, native, (2, 32), (4, 16))
+    case((32,), QuantValue.Q8S, packed, (2, 32), (4, 16))
+    case(None, QuantValue.Q8S, packed, (32,), (2, 16))
 
 
 def test_layout_ops_known_answers(dev, approx):
