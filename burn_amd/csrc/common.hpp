@@ -61,6 +61,13 @@ inline int value_qmax(int v) { return storage_value(v) == BQ_Q8S ? 127 : (storag
 inline int value_qmin(int v) { return -value_qmax(v) - (value_full(v) ? 1 : 0); }                                   // a
 inline float value_span(int v) { return static_cast<float>(value_qmax(v) - value_qmin(v)); }                        // b - a
 inline int num_quants(int v) { return 32 / value_bits(v); }
+// The Native store keeps one i8 per value whatever the value's width (QuantizedBytes::new,
+// crates/burn-std/src/tensor/quantization.rs:219-272; burn-store/src/tensor_snapshot.rs:545-557),
+// so a 4- or 2-bit tensor stored natively reads exactly like a Q8S one with small values: every
+// kernel that only reads values takes stored_value(). Quantizing to it clamps to the narrow range and
+// goes through the general kernels (fused_value() is false).
+inline int stored_value(int v, int store) { return store == BQ_STORE_NATIVE ? BQ_Q8S : v; }
+inline bool fused_value(int v, int store) { return value_known(v) && !(store == BQ_STORE_NATIVE && value_bits(v) != 8); }
 
 inline size_t round_up(size_t x, size_t a) { return (x + a - 1) / a * a; }
 

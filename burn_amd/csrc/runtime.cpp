@@ -94,7 +94,7 @@ static bq_status check_scheme(const bq_scheme& s, const size_t* shape, int rank,
   if (s.tensor_scale > 1 || (s.tensor_scale && s.level != BQ_LEVEL_BLOCK))
     BQ_FAIL(BQ_ERR_UNSUPPORTED_SCHEME, "a per-tensor scale on top (tensor_scale = %d) goes with block scales, as f32", s.tensor_scale);
   if (s.store == BQ_STORE_NATIVE) {
-    if (value_bits(s.value) != 8) BQ_FAIL(BQ_ERR_UNSUPPORTED_SCHEME, "Can't store native sub-byte values");
+    // one i8 per value, sub-byte values included (what the reference's CPU backend keeps and saves)
   } else if (s.store == BQ_STORE_PACKED_U32) {
     if (storable && shape[rank - 1] % static_cast<size_t>(num_quants(s.value)))
       BQ_FAIL(BQ_ERR_SHAPE, "Can't store in u32: last dim %zu is not a multiple of %d", shape[rank - 1],
@@ -814,7 +814,7 @@ static bq_status quantize_impl(const bq_tensor* x, const bq_scheme* scheme, cons
   // Run blocks with a fused kernel need no first pass: the largest block scale follows from the
   // tensor's absmax alone, and the block kernel splits each scale as it computes it.
   const long run = scheme->level == BQ_LEVEL_BLOCK ? run_block(*scheme, x->shape, x->rank) : 0;
-  if (two_level && dynamic && n > 0 && value_known(scheme->value) && run > 0 && run <= 512 &&
+  if (two_level && dynamic && n > 0 && fused_value(scheme->value, scheme->store) && run > 0 && run <= 512 &&
       fused_block_ok(static_cast<int>(run), scheme->value)) {
     uint32_t* cells = reinterpret_cast<uint32_t*>(q->scales() + q->num_scales);
     rc = bqk_absmax_f32(xin, n, cells, st);
@@ -887,8 +887,8 @@ static bq_status quantize_pass(const bq_tensor* x, const bq_scheme* scheme, bq_t
     }
     if (n == 0) break;
     const long run = run_block(*scheme, x->shape, x->rank);
-    if (!value_known(scheme->value)) {
-      // Q2S: the general kernels (any block shape). Per tensor, the range comes from the absmax
+    if (!fused_value(scheme->value, scheme->store)) {
+      // Q2S, and 4-bit values stored natively: the general kernels (any block shape). Per tensor, the range comes from the absmax
       // pass like every per-tensor quantize_dynamic.
       const bool per_tensor = scheme->level == BQ_LEVEL_TENSOR;
       if (per_tensor && dynamic) {
@@ -953,16 +953,17 @@ extern "C" bq_status bq_dequantize(const bq_tensor* q, int32_t float_dtype, bq_t
   const size_t n = q->numel();
   bq_status rc = BQ_OK;
   const long run = run_block(q->scheme, q->shape, q->rank);
+  const int qv = stored_value(q->scheme.value, q->scheme.store);  // (natively stored values read as 8-bit ones)
   if (n == 0) {
-  } else if (value_known(q->scheme.value) && run >= 0 &&
-             (run == 0 || (fused_block_ok(static_cast<int>(run), q->scheme.value) && run <= 512))) {
-    rc = bqk_dequantize(q->data, n, static_cast<int32_t>(run), q->scales(), q->scheme.value,
+  } else if (value_known(qv) && run >= 0 &&
+             (run == 0 || (fused_block_ok(static_cast<int>(run), qv) && run <= 512))) {
+    rc = bqk_dequantize(q->data, n, static_cast<int32_t>(run), q->scales(), qv,
                         q->scheme.store, float_dtype, f->data, st);
   } else {
     size_t blk[BQ_MAX_RANK];
     block_dims(q->scheme, q->rank, blk);
     rc = launch_dequantize_rect(q->data, q->shape, q->rank, q->scheme.level == BQ_LEVEL_TENSOR ? nullptr : blk,
-                                q->scales(), q->scheme.value, q->scheme.store, float_dtype, f->data, st);
+                                q->scales(), qv, q->scheme.store, float_dtype, f->data, st);
   }
   if (rc != BQ_OK) {
     bq_tensor_release(f);
@@ -1071,8 +1072,8 @@ static bq_status q_matmul_impl(const bq_tensor* lhs, const bq_tensor* rhs, int32
   // Fused path: float lhs x quantized rhs whose scales are per tensor or runs along N.
   // Ternary fast path (crates/burn-ndarray/src/ops/qtensor.rs:442-517): f32 activations times a
   // per-tensor Q2S 2-D weight, no bias, f32 out. Every other Q2S product dequantizes first.
-  if (!lq && rq && rhs->scheme.value == BQ_Q2S && rhs->scheme.level == BQ_LEVEL_TENSOR && lhs->dtype == BQ_F32 &&
-      out_dtype == BQ_F32 && rhs->rank == 2 && d.n % 16 == 0) {
+  if (!lq && rq && rhs->scheme.value == BQ_Q2S && rhs->scheme.store == BQ_STORE_PACKED_U32 &&
+      rhs->scheme.level == BQ_LEVEL_TENSOR && lhs->dtype == BQ_F32 && out_dtype == BQ_F32 && rhs->rank == 2 && d.n % 16 == 0) {
     bq_tensor* o = nullptr;
     BQ_TRY(new_float(dev, BQ_F32, d.out_shape, d.rank, &o));
     bq_status rc = launch_ternary_matmul(static_cast<const float*>(lhs->data), static_cast<const uint32_t*>(rhs->data),
@@ -1089,16 +1090,18 @@ static bq_status q_matmul_impl(const bq_tensor* lhs, const bq_tensor* rhs, int32
   // and then multiplied like a float one: the weight stays packed and the matrix-core kernels run.
   const int32_t lhs_dtype = lq ? target : lhs->dtype;
   long run = rq ? run_block(rhs->scheme, rhs->shape, rhs->rank) : -1;
-  bool fused = rq && run >= 0 && value_known(rhs->scheme.value);
+  // (natively stored values of any width are i8s: they multiply as Q8S ones)
+  const int rv = rq ? stored_value(rhs->scheme.value, rhs->scheme.store) : BQ_Q8S;
+  bool fused = rq && run >= 0 && value_known(rv);
   if (fused && run > 0) {
-    const size_t vpl = static_cast<size_t>(num_quants(rhs->scheme.value));
+    const size_t vpl = static_cast<size_t>(num_quants(rv));
     const size_t bw = static_cast<size_t>(run) / vpl;
     fused = (static_cast<size_t>(run) % vpl == 0) && bw && !(bw & (bw - 1)) && d.n % static_cast<size_t>(run) == 0;
   }
-  if (fused && (d.n % static_cast<size_t>(num_quants(rhs->scheme.value)))) fused = false;
+  if (fused && (d.n % static_cast<size_t>(num_quants(rv)))) fused = false;
   // (f32 activations, more than 32 rows: the fast kernels round to bf16; the device may ask for f32)
   if (fused && lhs_dtype == BQ_F32 && d.m > 32 && dev->f32_matmul_exact.load()) fused = false;
-  if (fused && !fused_matmul_ok(d.m, d.k, d.n, lhs_dtype, rhs->scheme.value,
+  if (fused && !fused_matmul_ok(d.m, d.k, d.n, lhs_dtype, rv,
                                 run > 0 ? d.n / static_cast<size_t>(run) : 0))
     fused = false;
   // The fused kernels take 16-byte aligned operands: with several batches every batch's slice of
@@ -1106,7 +1109,7 @@ static bq_status q_matmul_impl(const bq_tensor* lhs, const bq_tensor* rhs, int32
   if (fused && d.batches > 1) {
     const size_t vbytes = rhs->scheme.store == BQ_STORE_NATIVE
                               ? d.k * d.n
-                              : 4 * d.k * (d.n / static_cast<size_t>(num_quants(rhs->scheme.value)));
+                              : 4 * d.k * (d.n / static_cast<size_t>(num_quants(rv)));
     if ((d.m * d.k * dtype_size(lhs_dtype)) % 16 || (d.m * d.n * dtype_size(out_dtype)) % 16 || vbytes % 16 ||
         (run > 0 && (d.k * (d.n / static_cast<size_t>(run)) * sizeof(float)) % 16))
       fused = false;
@@ -1122,7 +1125,7 @@ static bq_status q_matmul_impl(const bq_tensor* lhs, const bq_tensor* rhs, int32
       if (lf) bq_tensor_release(lf);
       return rc;
     }
-    const size_t ws = bqk_q_matmul_workspace(d.m, d.k, d.n, lhs_dtype, rhs->scheme.value);
+    const size_t ws = bqk_q_matmul_workspace(d.m, d.k, d.n, lhs_dtype, rv);
     std::unique_lock<std::mutex> lock(dev->mu, std::defer_lock);
     if (ws) {
       lock.lock();  // the split-K workspace is shared by the calls on this device
@@ -1130,14 +1133,14 @@ static bq_status q_matmul_impl(const bq_tensor* lhs, const bq_tensor* rhs, int32
     }
     const size_t vbytes_per_batch = rhs->scheme.store == BQ_STORE_NATIVE
                                         ? d.k * d.n
-                                        : 4 * d.k * (d.n / static_cast<size_t>(num_quants(rhs->scheme.value)));
+                                        : 4 * d.k * (d.n / static_cast<size_t>(num_quants(rv)));
     const size_t scales_per_batch = run > 0 ? d.k * (d.n / static_cast<size_t>(run)) : 0;
     for (size_t b = 0; b < d.batches && rc == BQ_OK; ++b) {
       size_t lb, rb;
       batch_offsets(d, b, &lb, &rb);
       rc = bqk_q_linear(static_cast<char*>(l->data) + lb * d.m * d.k * dtype_size(lhs_dtype), lhs_dtype,
                         d.m, d.k, d.n, static_cast<char*>(rhs->data) + rb * vbytes_per_batch,
-                        rhs->scales() + rb * scales_per_batch, static_cast<int32_t>(run), rhs->scheme.value,
+                        rhs->scales() + rb * scales_per_batch, static_cast<int32_t>(run), rv,
                         rhs->scheme.store, bias, out_dtype,
                         static_cast<char*>(o->data) + b * d.m * d.n * dtype_size(out_dtype), dev->workspace,
                         dev->workspace_bytes, st);
@@ -1396,13 +1399,13 @@ static bq_status q_gather_impl(const bq_tensor* t, const int32_t* axes, const ui
   // Q8S words are the same bytes as native values, so a result whose last dim no longer fills whole
   // words is stored natively instead of being refused (the reference's CPU backend keeps one i8 per
   // value whatever the store says and permutes freely: ops/quantize.rs:406-431 of its tests ends
-  // with a last dim of 2). Sub-byte values have no native store: those results are refused.
+  // with a last dim of 2). Packed sub-byte values would have to be unpacked: those results are refused.
   if (scheme.store == BQ_STORE_PACKED_U32 && value_bits(scheme.value) == 8 && new_shape[rank - 1] % 4 != 0)
     scheme.store = BQ_STORE_NATIVE;
   bq_tensor* q = nullptr;
   BQ_TRY(new_quantized(t->dev, scheme, new_shape, rank, &q));  // also: "Can't store in u32" for the new last dim
   hipStream_t st = t->dev->stream;
-  bq_status rc = launch_q_gather(t->data, q->data, t->shape, rank, axes, flip, scheme.value,
+  bq_status rc = launch_q_gather(t->data, q->data, t->shape, rank, axes, flip, stored_value(scheme.value, scheme.store),
                                  scheme.store == BQ_STORE_NATIVE, st);
   if (rc == BQ_OK) {
     if (scheme.tensor_scale) {  // two-level: what the blob stores moves like the scales the kernels use

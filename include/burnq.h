@@ -76,7 +76,7 @@ enum { BQ_SCALE_F32 = 0, BQ_SCALE_F16 = 1, BQ_SCALE_BF16 = 2, BQ_SCALE_UE4M3 = 3
 typedef struct bq_scheme {
   uint8_t value;       /* BQ_Q8S | BQ_Q4S | BQ_Q2S | BQ_Q8F | BQ_Q4F | BQ_Q2F */
   uint8_t level;       /* BQ_LEVEL_TENSOR | BQ_LEVEL_BLOCK */
-  uint8_t store;       /* BQ_STORE_NATIVE (8-bit values only) | BQ_STORE_PACKED_U32 */
+  uint8_t store;       /* BQ_STORE_NATIVE (one i8 per value, whatever its width) | BQ_STORE_PACKED_U32 */
   uint8_t scale_dtype; /* BQ_SCALE_F32 | BQ_SCALE_F16 | BQ_SCALE_BF16 | BQ_SCALE_UE4M3 */
   uint8_t block_rank;
   uint8_t tensor_scale; /* block level only: 1 = an f32 per-tensor scale on top of the block scales (below) */
@@ -262,7 +262,8 @@ bq_status bq_q_reshape(const bq_tensor* t, const size_t* shape, int32_t rank, bq
  * dense tensor (the block of the scheme is permuted with the axes, so a [1, 32] block becomes
  * [32, 1] under a transpose). An axis out of bounds or repeated, which the reference panics on,
  * returns BQ_ERR_SHAPE, as does a packed sub-byte result whose last dim is not a whole number of
- * words (a Q8S result of that kind is stored natively: same bytes, one per value).
+ * words (a Q8S result of that kind is stored natively: same bytes, one per value; natively stored
+ * tensors of any value width permute freely).
  * q_flip flips the values and keeps every parameter where it is, block scales included, as the
  * reference does (burn-ndarray/src/ops/qtensor.rs:338-347): a value flipped into another block
  * is dequantized with that block's scale. */

@@ -87,6 +87,17 @@ def test_oversized_lds_request_is_refused_on_the_host():
     assert L.bqk_lds_request_status(64 * 1024 + 1, 64 * 1024) == _lib.ERR_HIP
 
 
+def test_data_len_of_natively_stored_values_of_any_width():
+    """crates/burn-store/src/tensor_snapshot.rs:545-581 (data_len_matches_materialized_bytes_when_
+    quantized): the reference's CPU backend stores quantized values natively, one i8 each, also for
+    4- and 2-bit value types, and a tensor's bytes are that many values plus its f32 scale -- for
+    element counts that are and are not multiples of 4."""
+    for value in (QuantValue.Q8S, QuantValue.Q4S, QuantValue.Q2S):
+        for shape in ((32, 32), (3, 3), (5, 5), (2, 3)):
+            n = shape[0] * shape[1]
+            assert ba.TensorData.data_len(shape, QuantScheme(value=value, store=QuantStore.Native)) == n + 4
+
+
 def test_data_len_refuses_what_q_from_data_would_refuse():
     """quantized_data_len runs the full scheme check: no division by a zero block extent, no
     length for a shape the scheme cannot hold."""
@@ -131,10 +142,10 @@ def test_scheme_supported_follows_the_reference_quantizable_rule():
     assert b"cannot absorb" in _lib.lib().bq_last_error()
     with pytest.raises(ValueError):          # a per-tensor scale narrower than f32 (refused where the scheme is built)
         base.per_block((4,), ScaleDtype.UE4M3).per_tensor(ScaleDtype.BF16)
-    # every value, packed; native only at 8 bits; rectangle blocks; unknown codes
+    # every value, packed or native (one i8 per value); rectangle blocks; unknown codes
     for v in QuantValue:
         assert QuantScheme(value=v).supported() and QuantScheme(value=v).per_block((2, 32)).supported()
-        assert QuantScheme(value=v, store=QuantStore.Native).supported() == (v.size_bits() == 8)
+        assert QuantScheme(value=v, store=QuantStore.Native).supported()
     c = base.to_c()
     c.value = 9
     assert _lib.lib().bq_scheme_supported(C.byref(c)) == _lib.ERR_UNSUPPORTED_SCHEME

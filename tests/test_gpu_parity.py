@@ -250,6 +250,37 @@ def test_reference_gpu_backend_quantize_dequantize_cases(dev):
         gpu_quantize_dynamic(dev, np.float32([[1.0, 6.35], [2.0, 3.0], [1.0, 3.0]]), QuantScheme(store=packed))
 
 
+@pytest.mark.parametrize("value", [QuantValue.Q4S, QuantValue.Q2S, QuantValue.Q4F, QuantValue.Q2F])
+@pytest.mark.parametrize("block", [None, (16,), (2, 8)])
+def test_sub_byte_values_stored_natively(dev, value, block):
+    """The reference's CPU backend keeps quantized values natively -- one i8 per value, 4- and 2-bit
+    value types included (crates/burn-std/src/tensor/quantization.rs:219-272 writes them that way,
+    :329-333 reads them back; burn-store/src/tensor_snapshot.rs:545-581 and
+    burn-store/tests/direct_writer.rs:76-93 save and size them) -- so a checkpoint written from it
+    holds such blobs. They quantize, serialise, load, dequantize, permute and multiply here like
+    any other tensor, bit for bit against the oracle; element counts that are not multiples of 4."""
+    scheme = QuantScheme(value=value, store=QuantStore.Native, block=block)
+    shape = (6, 16) if block else (5, 5)
+    x = awkward(shape, 77 + value.value)
+    tq, q_ref, s_ref, d_ref = check_quantize_dynamic(dev, x, scheme)
+    assert np.abs(q_ref).max() <= (8 if value.size_bits() == 4 else 2)
+    blob = QTensorOps.q_into_data(tq)
+    assert blob.bytes.size == x.size + 4 * s_ref.size == ba.TensorData.data_len(shape, scheme)
+    back = QTensorOps.q_from_data(blob, dev)
+    assert FloatOps.float_into_data(QTensorOps.dequantize(back)).tobytes() == d_ref.tobytes()
+    # static quantize against the same scales gives the same tensor
+    again = QTensorOps.quantize(FloatOps.float_from_data(x, dev), scheme, FloatOps.float_from_data(s_ref, dev))
+    assert QTensorOps.q_into_data(again).bytes.tobytes() == blob.bytes.tobytes()
+    if block is None:
+        t = QTensorOps.q_swap_dims(tq, 0, 1)
+        assert FloatOps.float_into_data(QTensorOps.dequantize(t)).tobytes() == np.ascontiguousarray(d_ref.T).tobytes()
+    # a product with it: lhs [3, rows] x tensor [rows, cols]
+    lhs = awkward((3, shape[0]), 5, outliers=False)
+    out = FloatOps.float_into_data(QTensorOps.q_matmul(FloatOps.float_from_data(lhs, dev), tq))
+    ref = lhs.astype(np.float64) @ d_ref.astype(np.float64)
+    assert np.abs(out - ref).max() <= 1e-5 * max(np.abs(ref).max(), 1e-30)
+
+
 # ------------------------------------------------------------------ seeded parity, all schemes
 
 @pytest.mark.parametrize("value", [QuantValue.Q8S, QuantValue.Q4S])
@@ -522,8 +553,8 @@ def test_error_behaviour(dev):
     x = FloatOps.float_from_data(np.zeros((4, 6), np.float32), dev)
     with pytest.raises(ba.BurnqError, match="Can't store in u32"):
         QTensorOps.quantize_dynamic(x, QuantScheme())                    # 6 % 4 != 0
-    with pytest.raises(ba.BurnqError, match="sub-byte"):
-        QTensorOps.quantize_dynamic(x, QuantScheme(value=QuantValue.Q4S, store=QuantStore.Native))
+    # (4-bit values stored natively, one i8 each, are what the reference's CPU backend keeps: accepted)
+    assert QTensorOps.quantize_dynamic(x, QuantScheme(value=QuantValue.Q4S, store=QuantStore.Native)).shape == (4, 6)
     x8 = FloatOps.float_from_data(np.zeros((4, 8), np.float32), dev)
     with pytest.raises(ba.BurnqError, match="evenly divisible"):
         QTensorOps.quantize_dynamic(x8, QuantScheme().per_block((3,)))
@@ -1190,13 +1221,14 @@ def test_q_matmul_with_full_range_weights(dev, value):
 
 # ------------------------------------------------------------------ random schemes
 
-def random_scheme_case(rng):
+def random_scheme_case(rng, native_any=False):
     """A quantizable (shape, scheme, magnitude): value, store, rank 1-4, per tensor or a block of rank
     1-rank with power-of-two extents (whole packed words along the last dim), any scale dtype, the
-    two-level form for f16 / ue4m3 block scales."""
+    two-level form for f16 / ue4m3 block scales. `native_any`: the Native store (one i8 per value) for
+    4- and 2-bit values too, as the reference's CPU backend keeps them."""
     value = [QuantValue.Q8S, QuantValue.Q4S, QuantValue.Q2S, QuantValue.Q8F, QuantValue.Q4F, QuantValue.Q2F][rng.integers(6)]
     nq = 32 // value.size_bits()
-    store = QuantStore.Native if nq == 4 and rng.integers(2) else QuantStore.PackedU32
+    store = QuantStore.Native if (nq == 4 or native_any) and rng.integers(2) else QuantStore.PackedU32
     rank = int(rng.integers(1, 5))
     sdt = [ScaleDtype.F32, ScaleDtype.F16, ScaleDtype.BF16, ScaleDtype.UE4M3][rng.integers(4)]
     block = None
@@ -1223,10 +1255,19 @@ def test_random_schemes_against_the_oracle(dev):
     """300 seeded cases over the whole scheme space: quantize_dynamic's blob, the dequantized floats
     and the blob round trip bit for bit, then one layout op (swap / permute / flip) on the result,
     whose dequantized values must be the same permutation of the source's."""
-    rng = np.random.default_rng(20240607)
+    scheme_sweep(dev, np.random.default_rng(20240607), 300, False, 60)
+
+
+def test_random_schemes_with_any_value_stored_natively(dev):
+    """150 more cases of the same sweep in which 4- and 2-bit values are stored natively half of the
+    time (one i8 per value: no word to fill, so any shape goes and every layout op applies)."""
+    scheme_sweep(dev, np.random.default_rng(515), 150, True, 40)
+
+
+def scheme_sweep(dev, rng, cases, native_any, distinct):
     seen = set()
-    for case in range(300):
-        shape, scheme, mag = random_scheme_case(rng)
+    for case in range(cases):
+        shape, scheme, mag = random_scheme_case(rng, native_any)
         x = (rng.standard_normal(shape) * mag).astype(np.float32)
         if rng.integers(5) == 0:
             x[rng.random(shape) < 0.3] = 0.0
@@ -1245,7 +1286,7 @@ def test_random_schemes_against_the_oracle(dev):
         rank = len(shape)
         axes = [int(a) for a in rng.permutation(rank)]
         nq = tq.scheme.num_quants()
-        if rank > 1 and (nq == 4 or shape[axes[-1]] % nq == 0):
+        if rank > 1 and (nq == 4 or scheme.store == QuantStore.Native or shape[axes[-1]] % nq == 0):
             tp = QTensorOps.q_permute(tq, axes)
             got = FloatOps.float_into_data(QTensorOps.dequantize(tp))
             assert got.tobytes() == np.ascontiguousarray(np.transpose(d, axes)).tobytes(), f"{label}: permute {axes}"
@@ -1253,7 +1294,7 @@ def test_random_schemes_against_the_oracle(dev):
         if scheme.block is None:   # (a flip keeps block scales in place: only per-tensor values commute with it)
             got = FloatOps.float_into_data(QTensorOps.dequantize(QTensorOps.q_flip(tq, fl)))
             assert got.tobytes() == np.ascontiguousarray(np.flip(d, fl)).tobytes(), f"{label}: flip {fl}"
-    assert len(seen) >= 60   # of the 80 (value, store) x (level, scale dtype, two-level) combinations
+    assert len(seen) >= distinct   # of the (value, store) x (level, scale dtype, two-level) combinations
 
 
 def test_random_matmuls_against_float64(dev):

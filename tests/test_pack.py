@@ -144,6 +144,13 @@ def test_quantized_entries_carry_the_blob_length(kats):
         e = r.find(f"t{i}")
         assert e["dtype"] == "QFloat" and e["data_offsets"][1] - e["data_offsets"][0] == case["len"]
         assert e["data_offsets"][0] % 256 == 0 and e["scheme"] == scheme
+    # crates/burn-store/tests/direct_writer.rs:76-93 (quantized_snapshot_writes_and_reads_back): a [5, 5]
+    # Q4S tensor as the reference's CPU backend holds it -- natively, one i8 per value: a sub-byte
+    # value type and a byte count (25 + 4) that is not a multiple of the scale alignment
+    s4 = QuantScheme(value=QuantValue.Q4S, store=QuantStore.Native)
+    blob = np.arange(29, dtype=np.uint8)
+    e = PackReader(PackWriter().add_bytes("weight", "QFloat", (5, 5), blob, scheme=s4).into_bytes()).find("weight")
+    assert tuple(e["shape"]) == (5, 5) and e["scheme"] == s4 and e["data_offsets"][1] - e["data_offsets"][0] == 29
     # a block scheme with 2-byte scales survives the scheme round trip too
     s2 = QuantScheme(store=QuantStore.Native).per_block((2, 16), ba.ScaleDtype.BF16)
     w2 = PackWriter().add_bytes("q", "QFloat", (4, 32), np.zeros(4 * 32 + 2 * 4, np.uint8), scheme=s2)
