@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the quantized-tensor hot path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-others] [--no-cpu] [--only c1,c3,c4,c5]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-others] [--no-cpu] [--only c1,c3,c4,c5,next,reference_bench]
 
 Prints ONE JSON line. The headline workload is block-32 Q8S PackedU32 quantize_dynamic +
 dequantize of an 8192x8192 f32 tensor (1 % outliers); a "step" is one such round trip with the
@@ -475,6 +475,57 @@ def run_c5(ba, dev, steps, warmup, cpu):
     return out
 
 
+def run_reference_bench(ba, dev, steps, warmup, cpu):
+    """The reference's own quantization benchmark (crates/burn-backend-tests/benches/quantization_ops.rs:
+    26-205): per-tensor Q8S, inputs (i % 1000) / 1000 - 0.5, 4K / 64K / 1M elements, every call
+    followed by a device sync (`bench_synced`) -- call latencies, not throughput. As there,
+    `quantize` builds the tensor from host data inside the timed call; `q_matmul` multiplies two
+    quantized n x n matrices. Medians of 200 calls, in microseconds."""
+    from burn_amd import FloatOps, QTensorOps, QuantScheme, QuantStore
+    from oracle import c_oracle as co
+    scheme = QuantScheme(store=QuantStore.Native)
+    osch = co.Scheme.make(co.Q8S, None, co.STORE_NATIVE)
+
+    def median_us(fn, reps=200):
+        for _ in range(10):
+            fn()
+            dev.sync()
+        t = []
+        for _ in range(reps):
+            t0 = time.perf_counter()
+            r = fn()
+            dev.sync()
+            t.append(time.perf_counter() - t0)
+            del r
+        return float(np.median(t) * 1e6)
+
+    def pattern(n):
+        return ((np.arange(n) % 1000).astype(np.float32) / np.float32(1000.0) - np.float32(0.5))
+
+    out = {"what": "call + device sync, median of 200, microseconds; the reference's published medians are its CPU backend's "
+                   "on another machine (BASELINE.md)", "scheme": "Q8S per tensor, Native store"}
+    for name, n in (("4K", 64 * 64), ("64K", 256 * 256), ("1M", 1024 * 1024)):
+        host = pattern(n)
+        x = FloatOps.float_from_data(host, dev)
+        q = QTensorOps.quantize_dynamic(x, scheme)
+        q_ref, s_ref = co.quantize_dynamic(host, osch)
+        values, scales = QTensorOps.q_into_data(q).split()
+        if values.tobytes() != q_ref.tobytes() or scales.tobytes() != s_ref.tobytes() or \
+                FloatOps.float_into_data(QTensorOps.dequantize(q)).tobytes() != co.dequantize(q_ref, osch, s_ref).tobytes():
+            raise ParityError(f"reference bench {name}: differs from the CPU oracle")
+        out[name] = {"quantize_with_upload_us": median_us(lambda: QTensorOps.quantize_dynamic(FloatOps.float_from_data(host, dev), scheme)),
+                     "quantize_us": median_us(lambda: QTensorOps.quantize_dynamic(x, scheme)),
+                     "dequantize_us": median_us(lambda: QTensorOps.dequantize(q))}
+    for n in (64, 256, 512):
+        host = pattern(n * n).reshape(n, n)
+        a = QTensorOps.quantize_dynamic(FloatOps.float_from_data(host, dev), scheme)
+        b = QTensorOps.quantize_dynamic(FloatOps.float_from_data(host, dev), scheme)
+        ad = FloatOps.float_into_data(QTensorOps.dequantize(a)).astype(np.float64)
+        matmul_gate(f"reference bench q_matmul {n}", FloatOps.float_into_data(QTensorOps.q_matmul(a, b)), ad @ ad)
+        out[f"q_matmul_{n}x{n}_us"] = median_us(lambda: QTensorOps.q_matmul(a, b))
+    return out
+
+
 # ------------------------------------------------------------------------------ CPU baseline
 
 def run_next(ba, dev, steps, warmup, cpu):
@@ -689,7 +740,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--no-others", action="store_true", help="skip the C1/C3/C4/C5 side measurements")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline legs")
-    ap.add_argument("--only", default="", help="comma list of side configs to run (c1,c3,c4,c5,next)")
+    ap.add_argument("--only", default="", help="comma list of side configs to run (c1,c3,c4,c5,next,reference_bench)")
     ap.add_argument("--c5-n", type=int, default=C5_N, help="weight columns of the C5 side measurement (default: C5's 14336)")
     args = ap.parse_args()
     C5_N = args.c5_n
@@ -742,7 +793,8 @@ def main():
     if not args.no_others:
         only = [s for s in args.only.split(",") if s]
         others = {}
-        for key, fn in (("c1", run_c1), ("c3", run_c3), ("c4", run_c4), ("c5", run_c5), ("next", run_next)):
+        for key, fn in (("c1", run_c1), ("c3", run_c3), ("c4", run_c4), ("c5", run_c5), ("next", run_next),
+                        ("reference_bench", run_reference_bench)):
             if only and key not in only:
                 continue
             log(f"{key} ...")

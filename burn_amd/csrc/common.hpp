@@ -87,11 +87,21 @@ struct bq_device {
   std::atomic<bool> validate{false};              // bq_device_set_validate
   std::atomic<bool> f32_matmul_exact{false};  // bq_device_set_f32_matmul_exact
   uint32_t* validate_cells = nullptr;             // 4 device counters of the validate mode
+  // Two pinned halves that host <-> device copies go through (lazily allocated, see upload()).
+  static constexpr size_t kStageBytes = 2u << 20;
+  std::mutex stage_mu;
+  char* stage[2] = {nullptr, nullptr};
+  hipEvent_t stage_ev[2] = {nullptr, nullptr};
 
   // *actual receives the size of the block handed out (at least `bytes`); pass it to release().
   bq_status alloc(size_t bytes, void** out, size_t* actual);  // stream-ordered reuse is safe: one stream
   void release(void* ptr, size_t bytes);
   bq_status ensure_workspace(size_t bytes);
+  // Blocking copies between pageable host memory and this device, behind the work already queued
+  // on the stream.
+  bq_status upload(void* dst, const void* src_host, size_t bytes);
+  bq_status download(void* dst_host, const void* src, size_t bytes);
+  bq_status ensure_stage();
   bq_status trim();
 };
 
