@@ -92,13 +92,16 @@ struct bq_device {
   std::mutex stage_mu;
   char* stage[2] = {nullptr, nullptr};
   hipEvent_t stage_ev[2] = {nullptr, nullptr};
+  bool stage_pending[2] = {false, false};         // a copy out of this half may still be in flight
+  int stage_next = 0;
 
   // *actual receives the size of the block handed out (at least `bytes`); pass it to release().
   bq_status alloc(size_t bytes, void** out, size_t* actual);  // stream-ordered reuse is safe: one stream
   void release(void* ptr, size_t bytes);
   bq_status ensure_workspace(size_t bytes);
-  // Blocking copies between pageable host memory and this device, behind the work already queued
-  // on the stream.
+  // Copies between pageable host memory and this device, behind the work already queued on the
+  // stream. upload() returns once the host buffer has been read (the transfer itself is stream
+  // ordered like a kernel); download() returns with the data in place.
   bq_status upload(void* dst, const void* src_host, size_t bytes);
   bq_status download(void* dst_host, const void* src, size_t bytes);
   bq_status ensure_stage();

@@ -292,18 +292,19 @@ bq_status bq_device::upload(void* dst, const void* src_host, size_t bytes) {
   BQ_TRY(ensure_stage());
   const char* src = static_cast<const char*>(src_host);
   char* to = static_cast<char*>(dst);
-  bool used[2] = {false, false};
-  int half = 0;
-  for (size_t off = 0; off < bytes; half ^= 1) {
+  for (size_t off = 0; off < bytes;) {
+    const int half = stage_next;
+    stage_next ^= 1;
     const size_t c = std::min(kStageBytes, bytes - off);
-    if (used[half]) BQ_HIP(hipEventSynchronize(stage_ev[half]));  // its previous chunk has left the buffer
+    if (stage_pending[half]) BQ_HIP(hipEventSynchronize(stage_ev[half]));  // its previous chunk has left the buffer
     std::memcpy(stage[half], src + off, c);
     BQ_HIP(hipMemcpyAsync(to + off, stage[half], c, hipMemcpyHostToDevice, stream));
     BQ_HIP(hipEventRecord(stage_ev[half], stream));
-    used[half] = true;
+    stage_pending[half] = true;
     off += c;
   }
-  BQ_HIP(hipStreamSynchronize(stream));
+  // (no synchronisation: the caller's buffer has been read, and whatever uses `dst` next is queued
+  // on the same stream behind the transfer)
   return BQ_OK;
 }
 
@@ -326,6 +327,7 @@ bq_status bq_device::download(void* dst_host, const void* src, size_t bytes) {
     issued += c;
     return BQ_OK;
   };
+  // (an upload still leaving a half is ahead of these transfers on the stream)
   BQ_TRY(fill(0));
   if (issued < bytes) BQ_TRY(fill(1));
   for (int h = 0; drained < bytes; h ^= 1) {
@@ -334,6 +336,7 @@ bq_status bq_device::download(void* dst_host, const void* src, size_t bytes) {
     drained += len[h];
     if (issued < bytes) BQ_TRY(fill(h));
   }
+  stage_pending[0] = stage_pending[1] = false;  // everything queued before the last transfer has finished
   return BQ_OK;
 }
 
@@ -624,7 +627,7 @@ extern "C" bq_status bq_float_from_data(bq_device* dev, const void* host, int32_
       bq_tensor_release(t);
       BQ_FAIL(BQ_ERR_NULL, "bq_float_from_data: null host buffer");
     }
-    const bq_status rc = dev->upload(t->data, host, t->value_bytes);  // (blocking: the host buffer is only borrowed)
+    const bq_status rc = dev->upload(t->data, host, t->value_bytes);  // (the host buffer is only borrowed: read before this returns)
     if (rc != BQ_OK) {
       bq_tensor_release(t);
       return rc;
