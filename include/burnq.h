@@ -170,7 +170,10 @@ size_t bq_tensor_num_scales(const bq_tensor* t);
 
 /* ------------------------------------------------------------------ float tensors
  * The slice of FloatTensorOps the path needs (float_from_data / float_into_data,
- * crates/burn-backend/src/backend/ops/tensor.rs). Row-major, contiguous. */
+ * crates/burn-backend/src/backend/ops/tensor.rs). Row-major, contiguous. A host buffer is only
+ * borrowed: bq_float_from_data / bq_q_from_data have read it when they return (the transfer to
+ * the device is then queued on the device's stream, ahead of every later call), and
+ * bq_float_into_data / bq_q_into_data return with the data in place. */
 bq_status bq_float_from_data(bq_device* dev, const void* host, int32_t dtype, const size_t* shape,
                              int32_t rank, bq_tensor** out);
 bq_status bq_float_into_data(const bq_tensor* t, void* host, size_t capacity_bytes);
