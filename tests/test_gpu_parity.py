@@ -549,6 +549,28 @@ def test_f32_matmul_exact_setting_removes_the_step_at_33_rows(dev, value):
     assert small <= 2e-5 and small == rel(QTensorOps.q_matmul(FloatOps.float_from_data(x[:32], dev), tq), ref[:32])
 
 
+def test_host_transfers_around_the_staging_size(dev):
+    """Host buffers travel through two pinned halves of 2 MiB: sizes just under, at and over one and
+    two halves, and far over, come back byte for byte, for float tensors and for quantized blobs
+    (values and scales in one copy or in two), also when uploads follow each other without a
+    synchronisation in between."""
+    half = 2 << 20
+    rng = np.random.default_rng(31)
+    sizes = [1, 3, half // 4 - 1, half // 4, half // 4 + 1, half // 2 + 5, 2 * half // 4, 2 * half // 4 + 7, 5 * half // 4 + 3]
+    held = []
+    for n in sizes:                       # n floats = 4 n bytes: 4 B ... 10 MiB + 12 B
+        x = rng.standard_normal(n).astype(np.float32)
+        held.append((x, FloatOps.float_from_data(x, dev)))   # back to back: no sync between uploads
+    for x, t in held:
+        assert FloatOps.float_into_data(t).tobytes() == x.tobytes()
+    for n in (half - 4, half, half + 4, 3 * half + 8):       # value bytes; scales behind them
+        scheme = QuantScheme(store=QuantStore.Native).per_block((4,))
+        blob = np.concatenate([rng.integers(-127, 128, n, dtype=np.int8).view(np.uint8),
+                               rng.random(n // 4, dtype=np.float32).view(np.uint8)])
+        t = QTensorOps.q_from_data(TensorData(blob, (n,), scheme), dev)
+        assert QTensorOps.q_into_data(t).bytes.tobytes() == blob.tobytes()
+
+
 def test_error_behaviour(dev):
     x = FloatOps.float_from_data(np.zeros((4, 6), np.float32), dev)
     with pytest.raises(ba.BurnqError, match="Can't store in u32"):
