@@ -106,6 +106,8 @@ SIGNATURES = {
     "bq_quantize": (_i32, [_vp, _ps, _vp, _pvp]),
     "bq_quantize_two_level": (_i32, [_vp, C.POINTER(CScheme), _vp, _vp, _pvp]),
     "bq_quantize_dynamic": (_i32, [_vp, _ps, _pvp]),
+    "bq_compute_range_abs_mean": (_i32, [_vp, _ps, _pvp]),
+    "bq_quantize_abs_mean": (_i32, [_vp, _ps, _pvp]),
     "bq_dequantize": (_i32, [_vp, _i32, _pvp]),
     "bq_q_matmul": (_i32, [_vp, _vp, _pvp]),
     "bq_q_matmul_as": (_i32, [_vp, _vp, _i32, _pvp]),

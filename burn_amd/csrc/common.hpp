@@ -155,6 +155,11 @@ bq_status launch_quantize_per_tensor(const float* x, size_t n, const float* scal
                                      hipStream_t stream);
 bq_status launch_quantize_run_block(const float* x, size_t n, int block, const float* scales_in, float* scales_out,
                                     int value, int store, void* values, int scale_dtype, hipStream_t stream);
+// Calibration::AbsMean: gamma = mean |x| per tensor (blk null; cells: BQ_ABSMAX_CELLS floats of scratch) or per
+// rectangle block; and compute_q_params on a symmetric range, scales[i] = (2 range[i]) / (b - a).
+bq_status launch_abs_mean(const float* x, const size_t* shape, int rank, const size_t* blk, float* cells, float* gamma,
+                          hipStream_t stream);
+bq_status launch_scales_from_range(const float* range, size_t n, int value, float* scales, hipStream_t stream);
 // dst[i] = scale_to_dtype(src[i]); f32 scales <-> their 2-byte wire form (f16 / bf16).
 bq_status launch_round_scales(const float* src, float* dst, size_t n, int scale_dtype, hipStream_t stream);
 // Two-level schemes. split: `scales` holds the f32 block scales of a quantize_dynamic and `cells` the

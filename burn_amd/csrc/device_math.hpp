@@ -166,12 +166,36 @@ __device__ __forceinline__ int unpack_field(uint32_t word, int j) {
   return static_cast<int>(word << (32 - BITS - j * BITS)) >> (32 - BITS);
 }
 
-// max over `width` consecutive lanes (width a power of two <= 64), result in every lane.
+// One DPP-modified move: every lane reads the lane that `CTRL` names inside its row of 16.
+template <int CTRL>
+__device__ __forceinline__ uint32_t dpp_lane(uint32_t v) {
+  return static_cast<uint32_t>(__builtin_amdgcn_update_dpp(0, static_cast<int>(v), CTRL, 0xF, 0xF, true));
+}
+
+// max of a non-negative float (an absmax) over `WIDTH` consecutive lanes (a power of two <= 64),
+// result in every lane. Non-negative floats order like their bit patterns, so every step is one
+// v_max_u32 whose second operand is fetched by DPP inside the vector ALU -- no LDS crossbar
+// (ds_bpermute), no canonicalising copies: quad_perm [1,0,3,2] and [2,3,0,1] inside a quad,
+// row_half_mirror across the quads of 8 lanes, row_mirror across the halves of a row of 16, then
+// v_permlane16_swap / v_permlane32_swap across rows and across the halves of the wave. max is
+// order-free, so the result is the one any other reduction order gives.
 template <int WIDTH>
-__device__ __forceinline__ float group_max(float v) {
-#pragma unroll
-  for (int off = WIDTH / 2; off > 0; off >>= 1) v = fmaxf(v, __shfl_xor(v, off, kWave));
-  return v;
+__device__ __forceinline__ float group_max(float f) {
+  static_assert(WIDTH >= 1 && WIDTH <= kWave && (WIDTH & (WIDTH - 1)) == 0, "a power of two up to the wave");
+  uint32_t v = __float_as_uint(f);
+  if (WIDTH >= 2) v = max(v, dpp_lane<0xB1>(v));    // quad_perm [1,0,3,2]
+  if (WIDTH >= 4) v = max(v, dpp_lane<0x4E>(v));    // quad_perm [2,3,0,1]
+  if (WIDTH >= 8) v = max(v, dpp_lane<0x141>(v));   // row_half_mirror
+  if (WIDTH >= 16) v = max(v, dpp_lane<0x140>(v));  // row_mirror
+  if (WIDTH >= 32) {  // rows 1, 3 of one copy <-> rows 0, 2 of the other
+    const auto r = __builtin_amdgcn_permlane16_swap(v, v, false, false);
+    v = max(r[0], r[1]);
+  }
+  if (WIDTH >= 64) {  // upper half of one copy <-> lower half of the other
+    const auto r = __builtin_amdgcn_permlane32_swap(v, v, false, false);
+    v = max(r[0], r[1]);
+  }
+  return __uint_as_float(v);
 }
 
 }  // namespace bq

@@ -631,6 +631,110 @@ bq_status launch_quantize_rect(const float* x, const size_t* shape, int rank, co
   return BQ_OK;
 }
 
+// ---- Calibration::AbsMean (crates/burn-backend/src/quantization/scheme.rs:57-69) ------------------
+// gamma = mean(|x|) per tensor or per block; the range is [-gamma, +gamma], so compute_q_params
+// gives scale = (2 gamma) / (b - a). The reference takes the mean with its float_mean / mean_dim
+// (a sum in an order of its backend's choosing, divided by the count); here every sum has a fixed
+// order, so results repeat run to run: per tensor, BQ_ABSMAX_CELLS workgroups each add the chunks
+// they stride over (a per-thread f32 sum, then the threads of the workgroup pairwise through LDS),
+// and one workgroup adds the cells in f64 and divides; per block, one thread adds its block's
+// elements in ascending order (rectangles of any shape; calibration runs once per weight).
+__device__ __forceinline__ float workgroup_sum(float v) {
+  __shared__ float part[kThreads];
+  part[threadIdx.x] = v;
+  __syncthreads();
+#pragma unroll
+  for (int half = kThreads / 2; half > 0; half >>= 1) {
+    if (static_cast<int>(threadIdx.x) < half) part[threadIdx.x] += part[threadIdx.x + half];
+    __syncthreads();
+  }
+  return part[0];
+}
+
+__global__ void __launch_bounds__(kThreads)
+abs_sum_kernel(const float* __restrict__ x, size_t n, float* __restrict__ cells) {
+  const size_t stride = static_cast<size_t>(gridDim.x) * kThreads;
+  float sum = 0.0f;
+  for (size_t i = static_cast<size_t>(blockIdx.x) * kThreads + threadIdx.x; i < n; i += stride) sum += fabsf(x[i]);
+  const float total = workgroup_sum(sum);
+  if (threadIdx.x == 0) cells[blockIdx.x] = total;
+}
+
+__global__ void __launch_bounds__(kThreads)
+abs_mean_from_cells_kernel(const float* __restrict__ cells, size_t n, float* __restrict__ gamma) {
+  __shared__ double part[kThreads];
+  double sum = 0.0;
+  for (int i = static_cast<int>(threadIdx.x); i < BQ_ABSMAX_CELLS; i += kThreads) sum += static_cast<double>(cells[i]);
+  part[threadIdx.x] = sum;
+  __syncthreads();
+  for (int half = kThreads / 2; half > 0; half >>= 1) {
+    if (static_cast<int>(threadIdx.x) < half) part[threadIdx.x] += part[threadIdx.x + half];
+    __syncthreads();
+  }
+  if (threadIdx.x == 0) gamma[0] = static_cast<float>(part[0] / static_cast<double>(n));
+}
+
+// One thread per block: mean |x| over the block rectangle.
+__global__ void rect_abs_mean_kernel(const float* __restrict__ x, RectDims d, size_t nblocks, size_t block_elems,
+                                     float* __restrict__ gamma) {
+  const size_t b = static_cast<size_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+  if (b >= nblocks) return;
+  size_t origin[BQ_MAX_RANK];
+  size_t rem = b;
+  for (int i = d.rank - 1; i >= 0; --i) {
+    origin[i] = (rem % d.grid[i]) * d.blk[i];
+    rem /= d.grid[i];
+  }
+  float sum = 0.0f;
+  for (size_t e = 0; e < block_elems; ++e) {
+    size_t r = e, idx = 0, stride = 1;
+    for (int i = d.rank - 1; i >= 0; --i) {
+      const size_t c = origin[i] + r % d.blk[i];
+      r /= d.blk[i];
+      idx += c * stride;
+      stride *= d.shape[i];
+    }
+    sum += fabsf(x[idx]);
+  }
+  gamma[b] = sum / static_cast<float>(block_elems);
+}
+
+// gamma[params] = mean |x| per tensor (blk null; `cells`: BQ_ABSMAX_CELLS floats of scratch) or per block.
+bq_status launch_abs_mean(const float* x, const size_t* shape, int rank, const size_t* blk, float* cells, float* gamma,
+                          hipStream_t st) {
+  size_t n = 1;
+  for (int i = 0; i < rank; ++i) n *= shape[i];
+  if (n == 0) return BQ_OK;
+  if (blk == nullptr) {
+    hipLaunchKernelGGL(abs_sum_kernel, dim3(BQ_ABSMAX_CELLS), dim3(kThreads), 0, st, x, n, cells);
+    BQ_HIP(hipGetLastError());
+    hipLaunchKernelGGL(abs_mean_from_cells_kernel, dim3(1), dim3(kThreads), 0, st, cells, n, gamma);
+    BQ_HIP(hipGetLastError());
+    return BQ_OK;
+  }
+  RectDims d{};
+  d.rank = rank;
+  size_t nblocks = 1, block_elems = 1;
+  for (int i = 0; i < rank; ++i) {
+    d.shape[i] = shape[i];
+    d.blk[i] = blk[i];
+    d.grid[i] = shape[i] / blk[i];
+    nblocks *= d.grid[i];
+    block_elems *= d.blk[i];
+  }
+  hipLaunchKernelGGL(rect_abs_mean_kernel, dim3((nblocks + 63) / 64), dim3(64), 0, st, x, d, nblocks, block_elems, gamma);
+  BQ_HIP(hipGetLastError());
+  return BQ_OK;
+}
+
+// scales[i] = (2 * range[i]) / (b - a) for any value type: compute_q_params on a symmetric range.
+bq_status launch_scales_from_range(const float* range, size_t n, int value, float* scales, hipStream_t st) {
+  if (n == 0) return BQ_OK;
+  hipLaunchKernelGGL(scales_from_absmax_kernel, dim3((n + 255) / 256), dim3(256), 0, st, range, n, value_span(value), scales);
+  BQ_HIP(hipGetLastError());
+  return BQ_OK;
+}
+
 // ---- scales in a 2-byte dtype ------------------------------------------------------------------
 // Tensors keep their scales as f32 on the device, holding values the scale dtype represents exactly
 // (rounded up at quantize time, or widened when a blob is loaded); the 2-byte form only exists on

@@ -286,7 +286,19 @@ bq_status bq_device::ensure_stage() {
   return BQ_OK;
 }
 
+// Host transfers go through the shared pinned halves and wait on events: recorded into a HIP graph
+// they would replay whatever the halves hold at that moment, so both are refused while the device's
+// stream is being captured (the header's rule for *_from_data / *_into_data, enforced).
+static bq_status refuse_while_capturing(bq_device* dev, const char* what) {
+  std::lock_guard<std::mutex> lock(dev->mu);
+  if (dev->cache.capturing())
+    BQ_FAIL(BQ_ERR_UNSUPPORTED_OP, "%s copies through host memory and cannot be recorded into a HIP graph: make it before "
+            "bq_graph_begin_capture or after bq_graph_end_capture", what);
+  return BQ_OK;
+}
+
 bq_status bq_device::upload(void* dst, const void* src_host, size_t bytes) {
+  BQ_TRY(refuse_while_capturing(this, "a host-to-device transfer (*_from_data)"));
   if (bytes == 0) return BQ_OK;
   std::lock_guard<std::mutex> lock(stage_mu);
   BQ_TRY(ensure_stage());
@@ -309,6 +321,7 @@ bq_status bq_device::upload(void* dst, const void* src_host, size_t bytes) {
 }
 
 bq_status bq_device::download(void* dst_host, const void* src, size_t bytes) {
+  BQ_TRY(refuse_while_capturing(this, "a device-to-host transfer (*_into_data)"));
   if (bytes == 0) {
     BQ_HIP(hipStreamSynchronize(stream));
     return BQ_OK;
@@ -725,44 +738,38 @@ extern "C" bq_status bq_q_from_data(bq_device* dev, const uint8_t* bytes, size_t
     bq_tensor_release(t);
     BQ_FAIL(BQ_ERR_NULL, "bq_q_from_data: null bytes");
   }
-  hipError_t e = hipSuccess;
   bq_status rc = BQ_OK;
   const bool two_level = scheme->tensor_scale != 0;
   // two-level: the block scales go to the stored copy, the kernels' scales are derived below
   float* const scales_dst = two_level ? t->wire_scales() : t->scales();
+  // (every transfer is a bq_device::upload: it has read the host bytes when it returns, is ordered on
+  // the stream like a kernel, and refuses to run inside a graph capture)
   if (!two_level && ssz == 4 && t->scales_offset == t->value_bytes) {
     // the device layout is the wire layout (values of a multiple of 256 bytes, f32 scales right
     // behind them): the whole blob arrives with one copy
     rc = dev->upload(t->data, bytes, need);
-    if (rc != BQ_OK) {
-      bq_tensor_release(t);
-      return rc;
+  } else {
+    rc = dev->upload(t->data, bytes, t->value_bytes);
+    if (rc == BQ_OK && ssz == 4) {
+      rc = dev->upload(scales_dst, bytes + t->value_bytes, 4 * t->num_scales);
+    } else if (rc == BQ_OK) {
+      // 2- and 1-byte scales: staged in a device block, widened (exactly) to the f32 the kernels read
+      void* stage = nullptr;
+      size_t stage_bytes = 0;
+      rc = dev->alloc(ssz * t->num_scales, &stage, &stage_bytes);
+      if (rc == BQ_OK) {
+        rc = dev->upload(stage, bytes + t->value_bytes, ssz * t->num_scales);
+        if (rc == BQ_OK) rc = launch_scales_from_wire(stage, scales_dst, t->num_scales, scheme->scale_dtype, dev->stream);
+        dev->release(stage, stage_bytes);  // (stream ordered: the next owner's work queues behind the kernel)
+      }
     }
-    *out = t;
-    return BQ_OK;
-  }
-  rc = dev->upload(t->data, bytes, t->value_bytes);
-  if (rc == BQ_OK && ssz == 4) {
-    rc = dev->upload(scales_dst, bytes + t->value_bytes, 4 * t->num_scales);
-  } else if (rc == BQ_OK) {
-    // 2- and 1-byte scales: staged in a device block, widened (exactly) to the f32 the kernels read
-    void* stage = nullptr;
-    size_t stage_bytes = 0;
-    rc = dev->alloc(ssz * t->num_scales, &stage, &stage_bytes);
-    if (rc == BQ_OK) {
-      e = hipMemcpyAsync(stage, bytes + t->value_bytes, ssz * t->num_scales, hipMemcpyHostToDevice, dev->stream);
-      if (e == hipSuccess) rc = launch_scales_from_wire(stage, scales_dst, t->num_scales, scheme->scale_dtype, dev->stream);
-      dev->release(stage, stage_bytes);  // (stream ordered: the next owner's work queues behind the kernel)
+    if (two_level && rc == BQ_OK) {
+      rc = dev->upload(t->wire_global(), bytes + t->value_bytes + ssz * t->num_scales, 4);
+      if (rc == BQ_OK) rc = launch_scales_times_global(t->wire_scales(), t->wire_global(), t->num_scales, t->scales(), dev->stream);
     }
   }
-  if (two_level && e == hipSuccess && rc == BQ_OK) {
-    e = hipMemcpyAsync(t->wire_global(), bytes + t->value_bytes + ssz * t->num_scales, 4, hipMemcpyHostToDevice, dev->stream);
-    if (e == hipSuccess) rc = launch_scales_times_global(t->wire_scales(), t->wire_global(), t->num_scales, t->scales(), dev->stream);
-  }
-  if (e == hipSuccess) e = hipStreamSynchronize(dev->stream);
-  if (e != hipSuccess || rc != BQ_OK) {
+  if (rc != BQ_OK) {
     bq_tensor_release(t);
-    if (e != hipSuccess) BQ_FAIL(BQ_ERR_HIP, "host to device copy failed: %s", hipGetErrorString(e));
     return rc;
   }
   *out = t;
@@ -781,23 +788,26 @@ extern "C" bq_status bq_q_into_data(const bq_tensor* t, uint8_t* bytes, size_t c
   hipStream_t st = t->dev->stream;
   const bool two_level = t->scheme.tensor_scale != 0;
   const float* const scales_src = two_level ? t->wire_scales() : t->scales();
-  if (two_level)  // the per-tensor scale comes last (every path below ends with a synchronisation)
-    BQ_HIP(hipMemcpyAsync(bytes + t->value_bytes + ssz * t->num_scales, t->wire_global(), 4, hipMemcpyDeviceToHost, st));
   if (!two_level && ssz == 4 && t->scales_offset == t->value_bytes) {  // dense on the device as on the wire: one copy
     return t->dev->download(bytes, t->data, need);
   }
+  // (every transfer below goes through bq_device::download, which returns with the bytes in place and
+  // refuses to run inside a graph capture; nothing is left in flight on an error return)
   BQ_TRY(t->dev->download(bytes, t->data, t->value_bytes));
-  if (ssz == 4) return t->dev->download(bytes + t->value_bytes, scales_src, 4 * t->num_scales);
-  void* stage = nullptr;
-  size_t stage_bytes = 0;
-  BQ_TRY(t->dev->alloc(ssz * t->num_scales, &stage, &stage_bytes));
-  bq_status rc = launch_scales_to_wire(scales_src, stage, t->num_scales, t->scheme.scale_dtype, st);
-  hipError_t e = hipSuccess;
-  if (rc == BQ_OK) e = hipMemcpyAsync(bytes + t->value_bytes, stage, ssz * t->num_scales, hipMemcpyDeviceToHost, st);
-  if (e == hipSuccess) e = hipStreamSynchronize(st);
-  t->dev->release(stage, stage_bytes);
-  if (e != hipSuccess) BQ_FAIL(BQ_ERR_HIP, "device to host copy failed: %s", hipGetErrorString(e));
-  return rc;
+  if (ssz == 4) {
+    BQ_TRY(t->dev->download(bytes + t->value_bytes, scales_src, 4 * t->num_scales));
+  } else {
+    void* stage = nullptr;
+    size_t stage_bytes = 0;
+    BQ_TRY(t->dev->alloc(ssz * t->num_scales, &stage, &stage_bytes));
+    bq_status rc = launch_scales_to_wire(scales_src, stage, t->num_scales, t->scheme.scale_dtype, st);
+    if (rc == BQ_OK) rc = t->dev->download(bytes + t->value_bytes, stage, ssz * t->num_scales);
+    t->dev->release(stage, stage_bytes);
+    if (rc != BQ_OK) return rc;
+  }
+  if (two_level)  // the per-tensor scale comes last
+    BQ_TRY(t->dev->download(bytes + t->value_bytes + ssz * t->num_scales, t->wire_global(), 4));
+  return BQ_OK;
 }
 
 // ================================================================================ quantize
@@ -1010,6 +1020,67 @@ extern "C" bq_status bq_quantize_two_level(const bq_tensor* x, const bq_scheme* 
 
 extern "C" bq_status bq_quantize_dynamic(const bq_tensor* x, const bq_scheme* scheme, bq_tensor** out) {
   return quantize_impl(x, scheme, nullptr, out);
+}
+
+// compute_range under Calibration::AbsMean (crates/burn-backend/src/quantization/scheme.rs:57-69).
+static bq_status abs_mean_impl(const bq_tensor* x, const bq_scheme* scheme, bq_tensor** gamma_out) {
+  BQ_NOTNULL(x);
+  BQ_NOTNULL(scheme);
+  BQ_NOTNULL(gamma_out);
+  *gamma_out = nullptr;
+  if (x->dtype != BQ_F32) BQ_FAIL(BQ_ERR_DTYPE, "compute_range takes an f32 tensor (got dtype %d)", x->dtype);
+  // (the reference's assert, scheme.rs:59-63)
+  if (scheme->tensor_scale != 0)
+    BQ_FAIL(BQ_ERR_UNSUPPORTED_SCHEME,
+            "AbsMean calibration has no two-level form: gamma is a mean over the whole tensor or block, which a "
+            "per-tensor scale cannot decompose");
+  BQ_TRY(check_scheme(*scheme, x->shape, x->rank, false));
+  const bool per_tensor = scheme->level == BQ_LEVEL_TENSOR;
+  size_t blk[BQ_MAX_RANK], pshape[BQ_MAX_RANK];
+  int prank = 1;
+  pshape[0] = 1;
+  if (!per_tensor) {
+    block_dims(*scheme, x->rank, blk);
+    prank = x->rank;
+    for (int i = 0; i < x->rank; ++i) pshape[i] = x->shape[i] / blk[i];
+  }
+  bq_tensor* gamma = nullptr;
+  BQ_TRY(new_float(x->dev, BQ_F32, pshape, prank, &gamma));
+  bq_tensor* cells = nullptr;
+  bq_status rc = BQ_OK;
+  if (per_tensor) {
+    const size_t ncells = BQ_ABSMAX_CELLS;
+    rc = new_float(x->dev, BQ_F32, &ncells, 1, &cells);
+  }
+  if (rc == BQ_OK && x->numel() == 0) rc = launch_fill_u32(static_cast<uint32_t*>(gamma->data), gamma->numel(), 0u, x->dev->stream);
+  if (rc == BQ_OK)
+    rc = launch_abs_mean(static_cast<const float*>(x->data), x->shape, x->rank, per_tensor ? nullptr : blk,
+                         cells ? static_cast<float*>(cells->data) : nullptr, static_cast<float*>(gamma->data), x->dev->stream);
+  if (cells) bq_tensor_release(cells);
+  if (rc != BQ_OK) {
+    bq_tensor_release(gamma);
+    return rc;
+  }
+  *gamma_out = gamma;
+  return BQ_OK;
+}
+
+extern "C" bq_status bq_compute_range_abs_mean(const bq_tensor* x, const bq_scheme* scheme, bq_tensor** gamma_out) {
+  return abs_mean_impl(x, scheme, gamma_out);
+}
+
+// The Quantizer's three steps (crates/burn-core/src/module/quantize.rs:47-49) with Calibration::AbsMean,
+// all on the device: gamma, scale = (2 gamma) / (b - a), quantize against it.
+extern "C" bq_status bq_quantize_abs_mean(const bq_tensor* x, const bq_scheme* scheme, bq_tensor** out) {
+  BQ_NOTNULL(out);
+  *out = nullptr;
+  bq_tensor* gamma = nullptr;
+  BQ_TRY(abs_mean_impl(x, scheme, &gamma));
+  bq_status rc = launch_scales_from_range(static_cast<const float*>(gamma->data), gamma->numel(), scheme->value,
+                                          static_cast<float*>(gamma->data), x->dev->stream);
+  if (rc == BQ_OK) rc = quantize_impl(x, scheme, gamma, out);
+  bq_tensor_release(gamma);
+  return rc;
 }
 
 // ================================================================================ dequantize

@@ -309,6 +309,24 @@ class QTensorOps:
         return _wrap(h, tensor.device)
 
     @staticmethod
+    def compute_range_abs_mean(tensor: Tensor, scheme: QuantScheme) -> Tensor:
+        """compute_range(scheme, tensor, Calibration::AbsMean) (crates/burn-backend/src/quantization/scheme.rs:57-69):
+        gamma = mean |x| per tensor or per block; the range is (-gamma, +gamma). Returns gamma."""
+        c = scheme.to_c()
+        h = C.c_void_p()
+        check(lib().bq_compute_range_abs_mean(tensor.handle, C.byref(c), C.byref(h)))
+        return _wrap(h, tensor.device)
+
+    @staticmethod
+    def quantize_abs_mean(tensor: Tensor, scheme: QuantScheme) -> Tensor:
+        """The Quantizer's compute_range -> compute_q_params -> quantize under Calibration::AbsMean
+        (crates/burn-core/src/module/quantize.rs:47-49)."""
+        c = scheme.to_c()
+        h = C.c_void_p()
+        check(lib().bq_quantize_abs_mean(tensor.handle, C.byref(c), C.byref(h)))
+        return _wrap(h, tensor.device)
+
+    @staticmethod
     def dequantize(tensor: Tensor, dtype: int = F32) -> Tensor:
         h = C.c_void_p()
         check(lib().bq_dequantize(tensor.handle, dtype, C.byref(h)))

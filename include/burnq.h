@@ -228,6 +228,18 @@ bq_status bq_quantize_two_level(const bq_tensor* x, const bq_scheme* scheme, con
  * scheme / two passes per tensor: scale = (2 * max|x|) / (b - a)
  * (crates/burn-backend/src/quantization/scheme.rs:44-104), then quantize as above. */
 bq_status bq_quantize_dynamic(const bq_tensor* x, const bq_scheme* scheme, bq_tensor** out);
+/* compute_range under Calibration::AbsMean (crates/burn-backend/src/quantization/scheme.rs:57-69; the
+ * calibration BitNet-style ternary weights are made with, crates/burn-std/src/tensor/quantization.rs:55-62):
+ * gamma = mean(|x|) over the tensor or over each block; the range is [-gamma, +gamma]. gamma_out is
+ * an f32 tensor of params_shape entries ([1], or dims / block) holding gamma, the range's maximum (its
+ * minimum is the negation). A two-level scheme is refused, as the reference asserts. The mean is a
+ * sum in a fixed order divided by the count (the reference's order is its backend's; its tests
+ * compare within Tolerance::default(), 0.5 %). */
+bq_status bq_compute_range_abs_mean(const bq_tensor* x, const bq_scheme* scheme, bq_tensor** gamma_out);
+/* What Quantizer::map_float does under Calibration::AbsMean (crates/burn-core/src/module/quantize.rs:47-49):
+ * compute_range -> compute_q_params -> quantize, i.e. scale = (2 gamma) / (b - a) -- gamma itself for
+ * the ternary Q2S -- and q = clamp(round(x / scale), a, b), without leaving the device. */
+bq_status bq_quantize_abs_mean(const bq_tensor* x, const bq_scheme* scheme, bq_tensor** out);
 /* QTensorOps::dequantize (qtensor.rs:152): x = (s == 0 ? 0.1 : s) * q, to BQ_F32 or BQ_BF16
  * (bf16 = f32 result rounded to nearest even, TensorData::convert_dtype). */
 bq_status bq_dequantize(const bq_tensor* q, int32_t float_dtype, bq_tensor** out);

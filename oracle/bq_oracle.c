@@ -140,6 +140,36 @@ int bqo_compute_range(const float* x, const size_t* shape, int rank, const bqo_s
   return 0;
 }
 
+/* compute_range(AbsMean): burn-backend/src/quantization/scheme.rs:57-69. gamma = mean(|x|) over the
+ * tensor (float_mean of float_abs) or over each block rectangle (reduce_blocks with float_mean_dim);
+ * the range is (-gamma, +gamma). The mean is a reassociable sum: the reference's order is its
+ * backend's, and its tests compare within Tolerance::default(). Here the sum is taken in binary64
+ * and rounded once, the value every f32 summation order approximates. */
+int bqo_compute_range_abs_mean(const float* x, const size_t* shape, int rank, const bqo_scheme* s,
+                               float* min_out, float* max_out) {
+  size_t n = num_elements(shape, rank);
+  if (n == 0) return -1;
+  if (s->level == BQO_LEVEL_TENSOR) {
+    double sum = 0.0;
+    for (size_t i = 0; i < n; ++i) sum += fabs((double)x[i]);
+    max_out[0] = (float)(sum / (double)n);
+    min_out[0] = -max_out[0];
+    return 0;
+  }
+  if (!divides(shape, rank, s)) return -1;
+  size_t nb = bqo_params_shape(shape, rank, s, NULL);
+  double* sums = (double*)calloc(nb ? nb : 1, sizeof(double));
+  if (!sums) return -1;
+  for (size_t i = 0; i < n; ++i) sums[bqo_block_of(shape, rank, s, i)] += fabs((double)x[i]);
+  const double per_block = (double)(n / nb);
+  for (size_t b = 0; b < nb; ++b) {
+    max_out[b] = (float)(sums[b] / per_block);
+    min_out[b] = -max_out[b];
+  }
+  free(sums);
+  return 0;
+}
+
 /* compute_q_params: burn-backend/src/quantization/scheme.rs:75-93. `mask_where(min_abs, mask,
  * max_abs)` takes max_abs where min_abs < max_abs, then `* 2` and `/ (b - a)` in f32. */
 void bqo_compute_q_params(const float* min, const float* max, size_t n, int value, float* scales) {

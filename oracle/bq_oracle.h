@@ -16,6 +16,8 @@
  *                        Q4S (-7,7): the 16 packed words <-> 128 values vector in
  *                        burn-std/src/tensor/quantization.rs:581-602 (it is quantize(arange(128))).
  *   bqo_compute_range    burn-backend-tests .../quantization/calibration.rs:7-59
+ *   bqo_compute_range_abs_mean  burn-backend-tests .../quantization/calibration.rs:62-125 (gamma 0.45 per
+ *                        tensor; 0.45 and 0.25 per block of 4)
  *   bqo_compute_q_params burn-backend-tests .../quantization/scheme.rs:9-49, ops/quantize.rs:171-206
  *   bqo_quantize         quantization.rs:164-199 (ndarray), ops/quantize.rs:25-93
  *   bqo_dequantize       quantization.rs:164-216 (exact assert_eq on the dequantized floats)
@@ -111,6 +113,10 @@ size_t bqo_block_of(const size_t* shape, int rank, const bqo_scheme* s, size_t i
 /* compute_range(MinMax): min and max per tensor or per block. Returns 0, -1 if not divisible. */
 int bqo_compute_range(const float* x, const size_t* shape, int rank, const bqo_scheme* s,
                       float* min_out, float* max_out);
+
+/* compute_range(AbsMean): gamma = mean |x| per tensor or per block; min = -gamma, max = +gamma. */
+int bqo_compute_range_abs_mean(const float* x, const size_t* shape, int rank, const bqo_scheme* s,
+                               float* min_out, float* max_out);
 
 /* compute_q_params: scale = (max(|min|,|max|) * 2) / (b - a), elementwise over n entries. */
 void bqo_compute_q_params(const float* min, const float* max, size_t n, int value, float* scales);

@@ -72,6 +72,7 @@ def lib():
         L.bqo_block_of.argtypes = [psz, i32, ps, sz]
         L.bqo_block_of.restype = sz
         L.bqo_compute_range.argtypes = [pf, psz, i32, ps, pf, pf]
+        L.bqo_compute_range_abs_mean.argtypes = [pf, psz, i32, ps, pf, pf]
         L.bqo_compute_q_params.argtypes = [pf, pf, sz, i32, pf]
         L.bqo_compute_q_params.restype = None
         L.bqo_quantize.argtypes = [pf, psz, i32, ps, pf, pi8]
@@ -151,6 +152,19 @@ def compute_range(x, scheme):
     if lib().bqo_compute_range(_p(x, C.c_float), sh, rank, C.byref(scheme),
                                _p(lo, C.c_float), _p(hi, C.c_float)):
         raise ValueError("shape not divisible by block")
+    return lo.reshape(pshape), hi.reshape(pshape)
+
+
+def compute_range_abs_mean(x, scheme):
+    """compute_range under Calibration::AbsMean: (-gamma, +gamma), gamma = mean |x| per tensor or block."""
+    x = np.ascontiguousarray(x, dtype=np.float32)
+    sh, rank = _shape(x.shape)
+    pshape, n = params_shape(x.shape, scheme)
+    lo = np.empty(n, np.float32)
+    hi = np.empty(n, np.float32)
+    if lib().bqo_compute_range_abs_mean(_p(x, C.c_float), sh, rank, C.byref(scheme),
+                                        _p(lo, C.c_float), _p(hi, C.c_float)):
+        raise ValueError("empty tensor or shape not divisible by block")
     return lo.reshape(pshape), hi.reshape(pshape)
 
 

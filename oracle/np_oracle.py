@@ -43,6 +43,19 @@ def compute_range(x, block=None):
     return v.min(axis=axes), v.max(axis=axes)
 
 
+def compute_range_abs_mean(x, block=None):
+    """compute_range(AbsMean) -- scheme.rs:57-69: gamma = mean |x| per tensor or per block rectangle,
+    range (-gamma, +gamma). The sum is taken in binary64 and rounded once."""
+    x = np.asarray(x, np.float32)
+    a = np.abs(x.astype(np.float64))
+    if block is None:
+        g = np.float32(a.mean()).reshape(1)
+    else:
+        v, axes = _split_view(a, block)
+        g = v.mean(axis=axes).astype(np.float32)
+    return -g, g
+
+
 def compute_q_params(lo, hi, value="Q8S"):
     """compute_q_params -- scheme.rs:75-93."""
     a, b = RANGES[value]

@@ -1440,6 +1440,178 @@ def test_burnpack_round_trip_of_device_tensors(dev, tmp_path):
         reader.load("layer.weight.q8_block", dev, scheme=QuantScheme(value=QuantValue.Q4S).per_block((32,)))
 
 
+def test_burnpack_container_written_by_the_reference(dev):
+    """tests/golden/mnist_model.bpk is examples/mnist-inference-web/model.bpk of the reference tree, a
+    container its own BurnpackWriter wrote (18 f32 tensors). Every tensor goes from the mapped file to
+    the device and comes back byte for byte; the two linear weights that fill whole blocks are then
+    quantized, written by this library's writer next to the originals, and read back."""
+    import os
+    from burn_amd import PackReader, PackWriter
+    path = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "mnist_model.bpk")
+    raw = open(path, "rb").read()
+    reader = PackReader(path)
+    assert len(reader) == 18
+    import struct
+    msize = struct.unpack("<IHI", raw[:10])[2]
+    start = (10 + msize + 255) // 256 * 256
+    loaded = {}
+    for e in reader.entries():
+        assert e["dtype"] == "F32"
+        begin, end = e["data_offsets"]
+        t = reader.load(e["name"], dev)
+        assert t.shape == tuple(e["shape"]) and t.dtype == ba.F32
+        back = FloatOps.float_into_data(t)
+        assert back.tobytes() == raw[start + begin:start + end], e["name"]
+        loaded[e["name"]] = (t, back)
+    # quantize what a Quantizer would (the linear weights), save, reload: blobs identical
+    writer = PackWriter()
+    for name, scheme in (("fc1.weight", QuantScheme().per_block((32,))), ("fc2.weight", QuantScheme(value=QuantValue.Q4S).per_block((32,)))):
+        t, host = loaded[name]
+        tq = QTensorOps.quantize_dynamic(t, scheme)
+        q_ref, s_ref = co.quantize_dynamic(host, oscheme(scheme))
+        blob = QTensorOps.q_into_data(tq).bytes
+        assert blob.tobytes() == co.encode(q_ref, oscheme(scheme), s_ref).tobytes()
+        writer.add_tensor(name, tq, param_id=reader.find(name)["param_id"])
+    again = PackReader(writer.into_bytes())
+    for name in ("fc1.weight", "fc2.weight"):
+        e = again.find(name)
+        assert e["dtype"] == "QFloat" and e["param_id"] == reader.find(name)["param_id"]
+        d = FloatOps.float_into_data(QTensorOps.dequantize(again.load(name, dev)))
+        assert np.abs(d - loaded[name][1]).max() <= np.abs(loaded[name][1]).max() / (127 if name == "fc1.weight" else 7)
+
+
+def test_burnpack_quantized_entry_of_another_producer(dev):
+    """A container assembled by hand whose dtype field is a `{"QFloat": <map>}` this library did not
+    write (serde's image of DType::QFloat(scheme); the scheme's own image is decided outside the
+    reference tree): the reader takes dtype, shape and bytes from the file, the scheme from the
+    caller, and the tensor equals what the oracle serialises."""
+    from test_pack import container
+    from burn_amd import PackReader
+    rng = np.random.default_rng(91)
+    x = (rng.standard_normal((64, 96)) * 0.05).astype(np.float32)
+    cases = {"q8": QuantScheme().per_block((32,)), "q4": QuantScheme(value=QuantValue.Q4S), "q8n": QuantScheme(store=QuantStore.Native).per_block((8, 16))}
+    foreign = {"QFloat": {"value": "Q8S", "mode": "Symmetric", "store": {"PackedNative": 3}, "level": {"Blocks": [7]}, "param": "F64"}}
+    blobs = {}
+    for name, scheme in cases.items():
+        q_ref, s_ref = co.quantize_dynamic(x, oscheme(scheme))
+        blobs[name] = (co.encode(q_ref, oscheme(scheme), s_ref), co.dequantize(q_ref, oscheme(scheme), s_ref))
+    raw = container([(name, foreign, x.shape, blobs[name][0].tobytes()) for name in cases])
+    reader = PackReader(raw)
+    for name, scheme in cases.items():
+        e = reader.find(name)
+        assert e["dtype"] == "QFloat" and e["scheme"] is None and tuple(e["shape"]) == x.shape
+        with pytest.raises(ba.BurnqError, match="pass the scheme"):
+            reader.load(name, dev)
+        t = reader.load(name, dev, scheme=scheme)
+        assert t.scheme == scheme and QTensorOps.q_into_data(t).bytes.tobytes() == blobs[name][0].tobytes()
+        assert FloatOps.float_into_data(QTensorOps.dequantize(t)).tobytes() == blobs[name][1].tobytes()
+
+
+# ------------------------------------------------------------------ Calibration::AbsMean
+
+def test_abs_mean_calibration_reference_cases(dev, kats, approx):
+    """crates/burn-backend-tests/tests/tensor/float/quantization/calibration.rs:62-125, with its
+    tolerance (Tolerance::default(): relative 0.005, absolute 1e-5), and the ternary weights the
+    Quantizer then makes of them."""
+    k = kats["abs_mean_calibration_per_tensor"]
+    scheme = QuantScheme(value=QuantValue.Q2S, store=QuantStore.Native)
+    g = FloatOps.float_into_data(QTensorOps.compute_range_abs_mean(FloatOps.float_from_data(np.float32(k["x"]), dev), scheme))
+    assert g.shape == (1,)
+    approx(g, k["expected_max"])
+    approx(-g, k["expected_min"])
+    tq = QTensorOps.quantize_abs_mean(FloatOps.float_from_data(np.float32(k["x"]), dev), scheme)
+    q, s = unpack_blob(QTensorOps.q_into_data(tq))
+    assert q.tolist() == [-1, -1, 0, 1]
+    approx(s.reshape(-1), k["expected_max"])
+    k = kats["abs_mean_calibration_per_block"]
+    scheme = QuantScheme(value=QuantValue.Q2S, store=QuantStore.Native).per_block(k["block"])
+    g = FloatOps.float_into_data(QTensorOps.compute_range_abs_mean(FloatOps.float_from_data(np.float32(k["x"]), dev), scheme))
+    assert g.shape == (2, 1)
+    approx(g, k["expected_max"])
+    # a two-level scheme is refused, as the reference asserts
+    two = QuantScheme().per_block((4,), ScaleDtype.F16).per_tensor()
+    with pytest.raises(ba.BurnqError, match="two-level"):
+        QTensorOps.compute_range_abs_mean(FloatOps.float_from_data(np.float32(k["x"]), dev), two)
+
+
+@pytest.mark.parametrize("value", [QuantValue.Q2S, QuantValue.Q8S, QuantValue.Q4S])
+@pytest.mark.parametrize("shape,block", [((4096,), None), ((257, 96), None), ((64, 128), (32,)), ((48, 64), (16, 16)),
+                                          ((6, 10, 32), (2, 5, 8)), ((1000, 1024), None), ((512, 512), (128,))])
+def test_abs_mean_calibration_against_the_oracle(dev, value, shape, block):
+    """gamma within 4 ulp-scale relative error (2e-6) of the oracle's binary64 mean -- the reference
+    compares within 0.5 % --, and the quantized tensor bit for bit what the oracle's quantize makes of
+    the scales the device derived (scale = 2 gamma / (b - a), one IEEE operation per step)."""
+    x = awkward(shape, 17 + len(shape))
+    store = QuantStore.Native if value == QuantValue.Q2S or shape[-1] % 8 else QuantStore.PackedU32
+    scheme = QuantScheme(value=value, store=store) if block is None else QuantScheme(value=value, store=store).per_block(block)
+    tx = FloatOps.float_from_data(x, dev)
+    g = FloatOps.float_into_data(QTensorOps.compute_range_abs_mean(tx, scheme))
+    lo_ref, g_ref = co.compute_range_abs_mean(x, oscheme(scheme))
+    assert g.shape == g_ref.shape
+    assert np.all(np.abs(g.astype(np.float64) - g_ref) <= 2e-6 * np.abs(g_ref)), float(np.abs(g - g_ref).max())
+    tq = QTensorOps.quantize_abs_mean(tx, scheme)
+    q, s = unpack_blob(QTensorOps.q_into_data(tq))
+    assert s.reshape(-1).tobytes() == co.compute_q_params(-g, g, VAL[value][0]).reshape(-1).tobytes()
+    q_ref = co.quantize(x, oscheme(scheme), s.reshape(g.shape))
+    assert (q == q_ref).all()
+    if value == QuantValue.Q2S:
+        assert set(np.unique(q).tolist()) == {-1, 0, 1}
+    # deterministic: the same bits on a second run
+    g2 = FloatOps.float_into_data(QTensorOps.compute_range_abs_mean(tx, scheme))
+    assert g2.tobytes() == g.tobytes()
+
+
+# ------------------------------------------------------------------ host threads
+
+def test_host_threads_share_one_device(dev):
+    """crates/burn-backend-tests/tests/tensor/multi_threads.rs: tensors used from several host
+    threads at once. Eight threads on one device, each running quantize_dynamic, dequantize and
+    q_matmul on its own inputs, repeatedly and concurrently; every result must equal, bit for bit,
+    what the same call gave on a single thread."""
+    import threading
+    rng = np.random.default_rng(404)
+    jobs = []
+    for t in range(8):
+        x = rng.standard_normal((64 + 8 * t, 256)).astype(np.float32)
+        w = (rng.standard_normal((256, 512)) * 0.02).astype(np.float32)
+        a = rng.standard_normal((1 + 5 * t, 256)).astype(np.float32)   # decode, split and tiled kernels
+        scheme = (QuantScheme().per_block((32,)), QuantScheme(value=QuantValue.Q4S).per_block((32,)), QuantScheme(store=QuantStore.Native))[t % 3]
+        jobs.append((x, w, a, scheme))
+
+    def run(job):
+        x, w, a, scheme = job
+        tq = QTensorOps.quantize_dynamic(FloatOps.float_from_data(x, dev), scheme)
+        blob = QTensorOps.q_into_data(tq).bytes.tobytes()
+        d = FloatOps.float_into_data(QTensorOps.dequantize(tq)).tobytes()
+        tw = QTensorOps.quantize_dynamic(FloatOps.float_from_data(w, dev), scheme)
+        y = FloatOps.float_into_data(QTensorOps.q_matmul(FloatOps.float_from_data(a, dev), tw)).tobytes()
+        return blob, d, y
+
+    expected = [run(j) for j in jobs]
+    for j, e in zip(jobs, expected):   # and the oracle agrees with the single-thread run
+        q_ref, s_ref = co.quantize_dynamic(j[0], oscheme(j[3]))
+        assert e[0] == co.encode(q_ref, oscheme(j[3]), s_ref).tobytes()
+    failures, barrier = [], threading.Barrier(8)
+
+    def worker(i):
+        try:
+            barrier.wait(timeout=60)
+            for rep in range(12):
+                got = run(jobs[i])
+                if got != expected[i]:
+                    failures.append((i, rep, [g == e for g, e in zip(got, expected[i])]))
+        except Exception as exc:   # noqa: BLE001
+            failures.append((i, repr(exc)))
+
+    threads = [threading.Thread(target=worker, args=(i,)) for i in range(8)]
+    for th in threads:
+        th.start()
+    for th in threads:
+        th.join(timeout=110)
+    assert not any(th.is_alive() for th in threads), "a worker thread did not finish"
+    assert not failures, failures[:3]
+
+
 # ------------------------------------------------------------------ the configs at full size
 
 def test_config1_per_tensor_q8s_native_4096(dev):

@@ -132,6 +132,46 @@ def test_calibration_ranges(kats):
     assert lo2.tolist() == lo.tolist() and hi2.tolist() == hi.tolist()
 
 
+def test_abs_mean_calibration_ranges(kats, approx):
+    """Calibration::AbsMean (scheme.rs:57-69) on the reference's own two cases (calibration.rs:62-125),
+    within the tolerance those tests use; C and numpy restatements agree; and what the arithmetic
+    fixes beyond them: gamma of a constant-magnitude tensor is that magnitude exactly, gamma is
+    invariant under sign flips and permutations inside a block, and for the ternary value the scale
+    compute_q_params derives from (-gamma, gamma) is gamma itself (2 gamma / 2)."""
+    k = kats["abs_mean_calibration_per_tensor"]
+    lo, hi = co.compute_range_abs_mean(f32(k["x"]), scheme("Q2S"))
+    approx(lo, k["expected_min"])
+    approx(hi, k["expected_max"])
+    lo2, hi2 = no.compute_range_abs_mean(f32(k["x"]))
+    assert lo2.tobytes() == lo.tobytes() and hi2.tobytes() == hi.tobytes()
+    k = kats["abs_mean_calibration_per_block"]
+    lo, hi = co.compute_range_abs_mean(f32(k["x"]), scheme("Q2S", block=k["block"]))
+    approx(lo, k["expected_min"])
+    approx(hi, k["expected_max"])
+    lo2, hi2 = no.compute_range_abs_mean(f32(k["x"]), k["block"])
+    assert lo2.tobytes() == lo.tobytes() and hi2.tobytes() == hi.tobytes()
+    # closed forms
+    rng = np.random.default_rng(5)
+    x = (rng.integers(0, 2, (6, 16)) * 2 - 1).astype(np.float32) * np.float32(0.375)
+    for block in (None, [2, 8], [16], [3, 4]):
+        lo, hi = co.compute_range_abs_mean(x, scheme("Q2S", block=block))
+        assert np.all(hi == np.float32(0.375)) and np.all(lo == np.float32(-0.375))
+    y = rng.standard_normal((4, 32)).astype(np.float32)
+    _, g = co.compute_range_abs_mean(y, scheme("Q2S", block=[32]))
+    _, g_flipped = co.compute_range_abs_mean(-y[:, ::-1], scheme("Q2S", block=[32]))
+    assert g.tobytes() == g_flipped.tobytes()
+    _, g_all = co.compute_range_abs_mean(y, scheme("Q2S"))
+    assert abs(float(g_all[0]) - float(np.abs(y.astype(np.float64)).mean())) <= 1e-7
+    s = co.compute_q_params(-g, g, co.Q2S)
+    assert s.tobytes() == g.tobytes()
+    # the ternary values that follow (BitNet's RoundClip(W / gamma, -1, 1)): the reference's own weights
+    # [-0.9, -0.3, 0, 0.6] / 0.45 = [-2, -0.67, 0, 1.33] -> [-1, -1, 0, 1]
+    w = f32(kats["abs_mean_calibration_per_tensor"]["x"])
+    _, gw = co.compute_range_abs_mean(w, scheme("Q2S"))
+    q = co.quantize(w, scheme("Q2S"), co.compute_q_params(-gw, gw, co.Q2S))
+    assert q.tolist() == [-1, -1, 0, 1]
+
+
 # ---------------------------------------------------------------- packing / wire format KATs
 
 def test_pack_i8s_to_u32(kats):

@@ -3,7 +3,9 @@ header constants and round trip (tests/header.rs), data-section alignment (tests
 reader rejections (tests/errors.rs) -- checked on the CPU against containers assembled by hand
 here, and the packed-Q4 byte lengths of crates/burn-store/src/tensor_snapshot.rs:517-541. The
 GPU round trip (device tensor -> file -> device tensor) is in test_gpu_parity.py."""
+import os
 import struct
+import subprocess
 
 import numpy as np
 import pytest
@@ -155,3 +157,106 @@ def test_quantized_entries_carry_the_blob_length(kats):
     s2 = QuantScheme(store=QuantStore.Native).per_block((2, 16), ba.ScaleDtype.BF16)
     w2 = PackWriter().add_bytes("q", "QFloat", (4, 32), np.zeros(4 * 32 + 2 * 4, np.uint8), scheme=s2)
     assert PackReader(w2.into_bytes()).find("q")["scheme"] == s2
+
+
+# ---- a container written by the reference -------------------------------------------------------
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+MNIST = os.path.join(ROOT, "tests", "golden", "mnist_model.bpk")
+# examples/mnist-inference-web/src/model.rs: two ConvBlocks (Conv2d [1, 64] and [64, 64], 3 x 3, with bias, + BatchNorm) and
+# three Linear layers 1600 -> 128 -> 128 -> 10, whose weights burn stores [d_input, d_output]
+MNIST_SHAPES = {
+    "conv1.conv.weight": (64, 1, 3, 3), "conv1.conv.bias": (64,), "conv2.conv.weight": (64, 64, 3, 3), "conv2.conv.bias": (64,),
+    **{f"conv{i}.norm.{p}": (64,) for i in (1, 2) for p in ("gamma", "beta", "running_mean", "running_var")},
+    "fc1.weight": (1600, 128), "fc1.bias": (128,), "fc2.weight": (128, 128), "fc2.bias": (128,), "fc3.weight": (128, 10), "fc3.bias": (10,),
+}
+
+
+def test_reads_a_container_written_by_the_reference():
+    """tests/golden/mnist_model.bpk is examples/mnist-inference-web/model.bpk of the reference tree,
+    written by burn's own BurnpackWriter: header, the 18 descriptors of that model (names, shapes,
+    dtypes, parameter ids), the layout rules (data section and every tensor on a 256-byte boundary,
+    tensors in file order without overlap), and sane contents."""
+    raw = open(MNIST, "rb").read()
+    magic, version, msize = struct.unpack("<IHI", raw[:10])
+    assert (magic, version) == (0x4255524E, 1) and raw[:4] == b"NRUB"
+    start = _lib.lib().bq_pack_data_section_start(msize)
+    assert start % 256 == 0 and start >= 10 + msize
+    for r in (PackReader(raw), PackReader(MNIST), PackReader(MNIST[:-4])):     # bytes, path, path without its extension
+        entries = r.entries()
+        assert len(r) == 18 and [e["name"] for e in entries] == sorted(MNIST_SHAPES)
+        spans = []
+        for e in entries:
+            assert e["dtype"] == "F32" and tuple(e["shape"]) == MNIST_SHAPES[e["name"]] and e["scheme"] is None
+            begin, end = e["data_offsets"]
+            assert begin % 256 == 0 and end - begin == 4 * int(np.prod(e["shape"])) and start + end <= len(raw)
+            assert e["param_id"] is not None and 0 < e["param_id"] < 2 ** 64
+            spans.append((begin, end))
+        assert len({e["param_id"] for e in entries}) == 18
+        spans.sort()
+        assert all(a_end <= b_begin for (_, a_end), (b_begin, _) in zip(spans, spans[1:]))
+        assert start + spans[-1][1] == len(raw)                                # the file ends with its last tensor
+    import ctypes as C
+    r = PackReader(raw)
+    for e in r.entries():
+        begin, end = e["data_offsets"]
+        data = np.frombuffer(C.string_at(e["data_ptr"], end - begin), np.float32)
+        assert data.tobytes() == raw[start + begin:start + end] and np.isfinite(data).all()
+        if e["name"].endswith("running_var"):
+            assert (data > 0).all()
+    # cutting the file anywhere inside its data section is refused (tests/errors.rs rejects_truncated_data_section)
+    for cut in (len(raw) - 1, len(raw) // 2, start + 1, start):
+        with pytest.raises(ba.BurnqError, match="smaller than its tensors"):
+            PackReader(raw[:cut])
+    for cut in (9, 10, 10 + msize - 1):
+        with pytest.raises(ba.BurnqError, match="InvalidHeader"):
+            PackReader(raw[:cut])
+
+
+def test_reader_limits_of_the_reference():
+    """crates/burn-pack/tests/errors.rs:19-66: an oversized metadata claim is refused before anything is
+    allocated for it, a metadata size past the end of the input is refused, and so is a version from
+    the future."""
+    header = lambda version, msize: struct.pack("<IHI", 0x4255524E, version, msize)   # noqa: E731
+    with pytest.raises(ba.BurnqError, match="exceeds the maximum"):
+        PackReader(header(1, 100 * 1024 * 1024 + 1))
+    PackReader(container([]))                                                         # an empty pack is fine (round_trip.rs empty_pack)
+    with pytest.raises(ba.BurnqError, match="InvalidHeader"):
+        PackReader(header(1, 4096))
+    with pytest.raises(ba.BurnqError, match="InvalidVersion"):
+        PackReader(header(2, 0))
+    # metadata made of a million one-byte items: refused by the node budget, not by the allocator
+    bomb = header(1, 8 << 20) + b"\x9a\x00\x7f\xff\xf0" + b"\x80" * ((8 << 20) - 5)
+    with pytest.raises(ba.BurnqError, match="MetadataDeserializationError"):
+        PackReader(bomb)
+
+
+def _sanitized(tmp_path, name, sources, lang):
+    exe = tmp_path / name
+    cc = ["g++", "-std=c++17"] if lang == "c++" else ["gcc", "-std=c11"]
+    subprocess.run(cc + ["-O1", "-g", "-fsanitize=address,undefined", "-fno-sanitize-recover=all", "-fno-omit-frame-pointer",
+                         "-I", os.path.join(ROOT, "include"), "-I", os.path.join(ROOT, "burn_amd", "csrc"), "-I", os.path.join(ROOT, "oracle")]
+                   + sources + ["-lm", "-o", str(exe)], check=True)
+    return str(exe)
+
+
+def test_container_parser_under_sanitizers_and_a_mutation_fuzz(tmp_path):
+    """The parser of untrusted containers (burn_amd/csrc/pack_format.hpp) built with the address and
+    undefined-behaviour sanitizers, fed 100 000 seeded mutations (bit flips, truncations, blown-up
+    lengths, nests) of valid containers, the reference-written one among them: every case is answered
+    with a status, and whatever is accepted describes bytes the container holds."""
+    exe = _sanitized(tmp_path, "fuzz_pack", [os.path.join(ROOT, "tests", "cpp", "fuzz_pack.cpp")], "c++")
+    out = subprocess.run([exe, "100000", "20250", MNIST], capture_output=True, text=True, timeout=600)
+    assert out.returncode == 0, out.stdout[-2000:] + out.stderr[-4000:]
+    assert "100000 cases" in out.stdout
+
+
+def test_oracle_and_block_cache_under_sanitizers(tmp_path):
+    """The C oracle and the allocator's block cache are host code too: both built with the address and
+    undefined-behaviour sanitizers and run over ragged shapes with exactly sized buffers."""
+    exe = _sanitized(tmp_path, "oracle_sanitize", [os.path.join(ROOT, "tests", "cpp", "oracle_sanitize.c"),
+                                                   os.path.join(ROOT, "oracle", "bq_oracle.c")], "c")
+    out = subprocess.run([exe], capture_output=True, text=True, timeout=300)
+    assert out.returncode == 0, out.stdout[-2000:] + out.stderr[-4000:]
+    exe = _sanitized(tmp_path, "test_block_cache", [os.path.join(ROOT, "tests", "cpp", "test_block_cache.cpp")], "c++")
+    out = subprocess.run([exe], capture_output=True, text=True, timeout=300)
+    assert out.returncode == 0, out.stdout[-2000:] + out.stderr[-4000:]

@@ -67,3 +67,81 @@ def test_static_scratch_refuses_products_beyond_its_size():
                                _lib.STORE_PACKED_U32, None, ba.F32, x.data_ptr, dev.stream)
     assert rc == _lib.ERR_SIZE
     dev.sync()
+
+
+def _static_call(L, dev, x, tw, bias, out, m, k, n, cval):
+    return L.bqk_q_linear_static(x.data_ptr, ba.F32, m, k, n, tw.data_ptr, tw.scales_ptr, 32, cval, _lib.STORE_PACKED_U32,
+                                 bias.data_ptr, ba.F32, out.data_ptr, dev.stream)
+
+
+def test_static_scratch_under_graph_capture_and_without_allocating():
+    """The two properties the entry point is for. (1) It allocates nothing: the device's free memory, as
+    hipMemGetInfo reports it, is the same before and after calls of every kernel family. (2) It can be
+    recorded into a HIP graph: the captured call, replayed three times with eager work and
+    synchronisations in between and fresh activations each time, gives the eager call's bytes."""
+    dev = ba.Device(0)
+    L = _lib.lib()
+    hip = C.CDLL("libamdhip64.so")
+    hip.hipMemGetInfo.argtypes = [C.POINTER(C.c_size_t), C.POINTER(C.c_size_t)]
+    rng = np.random.default_rng(77)
+
+    def free_bytes():
+        free, total = C.c_size_t(), C.c_size_t()
+        assert hip.hipMemGetInfo(C.byref(free), C.byref(total)) == 0
+        return free.value
+
+    for m, k, n, value in ((1, 1024, 2048, QuantValue.Q8S), (16, 2048, 4096, QuantValue.Q8S), (64, 2048, 1024, QuantValue.Q4S)):
+        cval = _lib.Q8S if value == QuantValue.Q8S else _lib.Q4S
+        w = (rng.standard_normal((k, n)) * 0.02).astype(np.float32)
+        tw = QTensorOps.quantize_dynamic(FloatOps.float_from_data(w, dev), QuantScheme(value=value).per_block((32,)))
+        bias = FloatOps.float_from_data(rng.standard_normal(n).astype(np.float32), dev)
+        xs = [rng.standard_normal((m, k)).astype(np.float32) for _ in range(3)]
+        x = FloatOps.float_from_data(xs[0], dev)
+        out = FloatOps.float_empty((m, n), dev)
+        eager = []
+        for xh in xs:      # eager results for the three activations (also warms every code path)
+            x = FloatOps.float_from_data(xh, dev)
+            _lib.check(_static_call(L, dev, x, tw, bias, out, m, k, n, cval))
+            eager.append(FloatOps.float_into_data(out).tobytes())
+        dev.sync()
+        before = free_bytes()
+        for _ in range(4):
+            _lib.check(_static_call(L, dev, x, tw, bias, out, m, k, n, cval))
+        dev.sync()
+        assert free_bytes() == before, "the allocation-free entry point changed the device's free memory"
+        # captured: the graph reads `xin` and writes `gout`; both live outside the capture
+        xin = FloatOps.float_from_data(xs[0], dev)
+        gout = FloatOps.float_empty((m, n), dev)
+        graph, rc = dev.capture(lambda: _static_call(L, dev, xin, tw, bias, gout, m, k, n, cval))
+        assert rc == _lib.OK
+        for rep, xh in enumerate(xs):
+            # eager work between the replays: new activations copied into the graph's input, a sync
+            tmp = FloatOps.float_from_data(xh, dev)
+            _lib.check(L.bqk_copy(tmp.data_ptr, xin.data_ptr, m * k * 4, dev.stream))
+            dev.sync()
+            graph.launch()
+            got = FloatOps.float_into_data(gout).tobytes()
+            assert got == eager[rep], f"replay {rep} of the captured static call differs (m={m})"
+    dev.sync()
+
+
+def test_host_transfers_are_refused_while_capturing():
+    """*_from_data / *_into_data go through pinned staging memory and wait on events; recorded into a
+    graph they would replay stale bytes, so they fail loudly instead (and the capture still ends cleanly)."""
+    dev = ba.Device(0)
+    t = FloatOps.float_from_data(np.arange(64, dtype=np.float32), dev)
+    seen = {}
+
+    def body():
+        for name, fn in (("from_data", lambda: FloatOps.float_from_data(np.ones(64, np.float32), dev)),
+                         ("into_data", lambda: FloatOps.float_into_data(t))):
+            try:
+                fn()
+                seen[name] = None
+            except ba.BurnqError as e:
+                seen[name] = e.status
+    graph, _ = dev.capture(body)
+    assert seen == {"from_data": _lib.ERR_UNSUPPORTED_OP, "into_data": _lib.ERR_UNSUPPORTED_OP}
+    del graph
+    assert FloatOps.float_into_data(t).tolist() == list(range(64))
+    dev.sync()
