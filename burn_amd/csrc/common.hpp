@@ -71,6 +71,12 @@ inline bool fused_value(int v, int store) { return value_known(v) && !(store == 
 
 inline size_t round_up(size_t x, size_t a) { return (x + a - 1) / a * a; }
 
+// Ticket counters of the single-launch split-K sum (splitk_tail.hpp): one counter per column tile
+// of a launch, a 128-byte line apart.
+constexpr unsigned kTicketStride = 32;     // words between two tiles' counters
+constexpr unsigned kTicketCells = 2048;    // tiles a launch may have
+constexpr size_t kTicketBytes = static_cast<size_t>(kTicketCells) * kTicketStride * sizeof(unsigned);
+
 }  // namespace bq
 
 // ---- opaque types ----------------------------------------------------------------------------
@@ -82,6 +88,7 @@ struct bq_device {
   bq::BlockCache cache;                           // cached allocations, graph-capture bookkeeping
   void* workspace = nullptr;                      // split-K partials, bf16 copy of an f32 lhs
   size_t workspace_bytes = 0;
+  unsigned* tickets = nullptr;                    // counters of the single-launch split-K sum (zero between launches)
   int num_cus = 256;
   size_t lds_limit = 64 * 1024;                   // largest dynamic LDS request a launch may make
   std::atomic<bool> validate{false};              // bq_device_set_validate
@@ -231,7 +238,14 @@ bq_status configure_dynamic_lds(const void* kernel, size_t bytes, const char* wh
 
 // Device address of the static scratch array of bqk_q_linear_static on the current device
 // (qmatmul.hip): resolved once per device.
-bq_status static_scratch_ptr(void** out);
+bq_status static_scratch_ptr(void** out, unsigned** tickets_out = nullptr);
+// bqk_q_linear plus the ticket counters that let the split-K kernels finish their own sum in one
+// launch (qmatmul.hip, splitk_tail.hpp): `tickets` is kTicketBytes of device memory, zero between
+// launches; calls sharing it must not overlap on the device.
+bq_status q_linear_with_tickets(const void* x, int32_t x_dtype, size_t m, size_t k, size_t n, const void* w_values,
+                                const float* w_scales, int32_t block, int32_t value, int32_t store, const float* bias,
+                                int32_t out_dtype, void* out, void* workspace, size_t workspace_bytes, unsigned* tickets,
+                                void* stream);
 
 // Counts, over n floats, NaNs into counts[0] and infinities into counts[1] (device u32 cells that
 // the kernel adds to; quantize.hip). Used by the validate mode.

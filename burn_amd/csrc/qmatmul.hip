@@ -24,6 +24,7 @@
 
 #include "common.hpp"
 #include "device_math.hpp"
+#include "splitk_tail.hpp"
 
 namespace bq {
 
@@ -169,7 +170,8 @@ template <int VPL, bool PER_TENSOR, int M, bool X_BF16 = false>
 __global__ void __launch_bounds__(gemv1_waves(VPL, M) * kWave)
 qgemv1_kernel(const void* __restrict__ x, const uint32_t* __restrict__ w,
               const float* __restrict__ scales, size_t K, size_t NQ, unsigned scale_shift,
-              size_t scales_per_row, size_t rows_per_wg, float* __restrict__ part) {
+              size_t scales_per_row, size_t rows_per_wg, float* __restrict__ part,
+              unsigned* __restrict__ tickets, const float* __restrict__ bias, int out_bf16, void* __restrict__ out) {
   constexpr int WPL = gemv1_words(VPL);
   constexpr int CPL = WPL * VPL;  // columns per lane: 16
   typedef uint32_t LoadT __attribute__((ext_vector_type(WPL)));  // one 16- or 8-byte load
@@ -300,9 +302,17 @@ qgemv1_kernel(const void* __restrict__ x, const uint32_t* __restrict__ w,
       float v = red[0][at];
 #pragma unroll
       for (int ww = 1; ww < WAVES; ++ww) v += red[ww][at];
-      if (n_base + o < N) dst[o] = v;
+      if (n_base + o < N) {
+        // (one launch: the partials are read by another workgroup, possibly on another XCD)
+        if (tickets != nullptr) __hip_atomic_store(dst + o, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        else dst[o] = v;
+      }
     }
   }
+  // tickets: the last workgroup to finish a column strip sums the K slices and writes the output
+  if (tickets != nullptr)
+    splitk_reduce_tail<THREADS>(part, tickets + static_cast<size_t>(blockIdx.x) * kTicketStride, gridDim.y, M, N, n_base,
+                                static_cast<unsigned>(N - n_base < ELEMS ? N - n_base : ELEMS), bias, out_bf16 != 0, out);
 }
 
 // out[i] = sum over slices of part[s][i]. A workgroup owns 256 / SL float4 columns; its SL "slice
@@ -715,7 +725,10 @@ __global__ void empty_k_kernel(const float* __restrict__ bias, size_t mn, size_t
 static bq_status q_matmul_core(const void* lhs, int32_t lhs_dtype, size_t m, size_t k, size_t n,
                                const void* w_values, const float* w_scales, int32_t block,
                                int32_t value, int32_t store, const float* bias, int32_t out_dtype, void* out,
-                               void* workspace, size_t workspace_bytes, void* stream, size_t* need_out = nullptr) {
+                               void* workspace, size_t workspace_bytes, void* stream, size_t* need_out = nullptr,
+                               unsigned* tickets = nullptr) {
+  // tickets: kTicketBytes of device memory, zero between launches (splitk_tail.hpp), or null. With
+  // them the decode kernel finishes its own split-K sum for one or two rows: one launch instead of two.
   // need_out: dry run. The arguments are validated and the kernel is chosen as usual, but nothing is
   // launched: *need_out receives the scratch bytes that kernel would use.
   if (need_out) *need_out = 0;
@@ -768,6 +781,9 @@ static bq_status q_matmul_core(const void* lhs, int32_t lhs_dtype, size_t m, siz
       BQ_FAIL(BQ_ERR_SIZE, "q_matmul workspace: need %zu bytes, got %zu", need, workspace_bytes);
     float* part = static_cast<float*>(workspace);
     unsigned slices = 0;
+    // (the single-launch sum does not pay here: with 3 to 32 rows the partial sums are megabytes, which
+    // the reduction kernel reads with the whole chip while a last workgroup per tile would read them
+    // alone -- measured on the 4096 x 14336 weight, M = 4 / 16: 20.1 / 25.3 us against 19.8 / 22.5 us)
     BQ_TRY(launch_qsplit(lhs, lhs_dtype, w, w_scales, m, k, n, value, block, part, &slices, st));
     return launch_gemv_reduce(part, m * n, slices, bias, n, out_dtype, out, st);
   }
@@ -784,22 +800,26 @@ static bq_status q_matmul_core(const void* lhs, int32_t lhs_dtype, size_t m, siz
     const size_t nq = n / cpl;
     const unsigned shift = per_tensor ? 0 : log2_exact(static_cast<size_t>(block) / cpl);
     dim3 grid(p.strips, p.slices), tb(gemv1_waves(static_cast<int>(vpl), static_cast<int>(m)) * kWave);
+    // One launch when the caller brought ticket counters, for one or two rows: the last workgroup of a
+    // strip reads slices x M x 4 KiB of partial sums by itself, which is less than a second launch costs
+    // (4096 x 14336 weight, M = 1: 15.7 against 16.05 us per product) only while M is small.
+    unsigned* const tk = (tickets != nullptr && m <= 2 && p.strips <= kTicketCells && need < 0x7FFFFFFFull) ? tickets : nullptr;
     const void* x = lhs;
     const uint32_t* w4 = static_cast<const uint32_t*>(w_values);
 #define BQ_GEMV1B(V, MM)                                                                                         \
   if (per_tensor)                                                                                                \
     hipLaunchKernelGGL((qgemv1_kernel<V, true, MM, true>), grid, tb, 0, st, x, w4, w_scales, k, nq, shift, spr,  \
-                       p.rows_per_slice, part);                                                                  \
+                       p.rows_per_slice, part, tk, bias, out_dtype == BQ_BF16, out);                             \
   else                                                                                                           \
     hipLaunchKernelGGL((qgemv1_kernel<V, false, MM, true>), grid, tb, 0, st, x, w4, w_scales, k, nq, shift, spr, \
-                       p.rows_per_slice, part)
+                       p.rows_per_slice, part, tk, bias, out_dtype == BQ_BF16, out)
 #define BQ_GEMV1(V, MM)                                                                                    \
   if (per_tensor)                                                                                          \
     hipLaunchKernelGGL((qgemv1_kernel<V, true, MM>), grid, tb, 0, st, x, w4, w_scales, k, nq, shift, spr,  \
-                       p.rows_per_slice, part);                                                            \
+                       p.rows_per_slice, part, tk, bias, out_dtype == BQ_BF16, out);                       \
   else                                                                                                     \
     hipLaunchKernelGGL((qgemv1_kernel<V, false, MM>), grid, tb, 0, st, x, w4, w_scales, k, nq, shift, spr, \
-                       p.rows_per_slice, part)
+                       p.rows_per_slice, part, tk, bias, out_dtype == BQ_BF16, out)
     if (lhs_dtype == BQ_BF16) {  // m is 1 or 2
       if (value == BQ_Q8S) {
         if (m == 1) { BQ_GEMV1B(4, 1); } else { BQ_GEMV1B(4, 2); }
@@ -828,6 +848,7 @@ static bq_status q_matmul_core(const void* lhs, int32_t lhs_dtype, size_t m, siz
 #undef BQ_GEMV1
 #undef BQ_GEMV1B
     BQ_HIP(hipGetLastError());
+    if (tk != nullptr) return BQ_OK;
     return launch_gemv_reduce(part, m * n, p.slices, bias, n, out_dtype, out, st);
   }
 
@@ -918,6 +939,20 @@ extern "C" bq_status bqk_q_linear(const void* x, int32_t x_dtype, size_t m, size
                        workspace, workspace_bytes, stream);
 }
 
+namespace bq {
+// bqk_q_linear with the ticket counters of the single-launch split-K sum (the handle level passes its
+// device context's; kTicketBytes, zero between launches, one call at a time per device).
+bq_status q_linear_with_tickets(const void* x, int32_t x_dtype, size_t m, size_t k, size_t n, const void* w_values,
+                                const float* w_scales, int32_t block, int32_t value, int32_t store, const float* bias,
+                                int32_t out_dtype, void* out, void* workspace, size_t workspace_bytes, unsigned* tickets,
+                                void* stream) {
+  if (bias != nullptr && (reinterpret_cast<uintptr_t>(bias) & 15u))
+    BQ_FAIL(BQ_ERR_SHAPE, "q_linear bias must be 16-byte aligned");
+  return q_matmul_core(x, x_dtype, m, k, n, w_values, w_scales, block, value, store, bias, out_dtype, out,
+                       workspace, workspace_bytes, stream, nullptr, tickets);
+}
+}  // namespace bq
+
 // ================================================================================ no allocation
 // bqk_q_linear for callers that cannot allocate (code under HIP graph capture, serving loops,
 // harnesses that forbid hipMalloc): the split-K partials and the bf16 copy of an f32 lhs, which
@@ -926,13 +961,18 @@ extern "C" bq_status bqk_q_linear(const void* x, int32_t x_dtype, size_t m, size
 // until the process ends; the address is looked up once per device and the kernels only ever see
 // that pointer (the array's name is a host-side stand-in, not a device address).
 static __device__ __align__(256) unsigned char scratch[BQK_STATIC_SCRATCH_BYTES];
+// The ticket counters of its single-launch split-K sum: zero when the module is loaded, left zero by
+// every launch (splitk_tail.hpp). Like `scratch`, shared by all calls on one GPU.
+static __device__ __align__(256) unsigned static_tickets[kTicketCells * kTicketStride];
 
 namespace bq {
 
-// The device address of `scratch` on the current device (looked up on first use, then cached).
-bq_status static_scratch_ptr(void** out) {
+// The device address of `scratch` on the current device (looked up on first use, then cached), and
+// of the ticket counters beside it.
+bq_status static_scratch_ptr(void** out, unsigned** tickets_out) {
   static std::mutex mu;
   static void* ptrs[64] = {nullptr};
+  static unsigned* tickets[64] = {nullptr};
   int ordinal = 0;
   BQ_HIP(hipGetDevice(&ordinal));
   if (ordinal < 0 || ordinal >= 64) BQ_FAIL(BQ_ERR_HIP, "device ordinal %d out of range", ordinal);
@@ -942,9 +982,15 @@ bq_status static_scratch_ptr(void** out) {
     BQ_HIP(hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)));
     if (p == nullptr || (reinterpret_cast<uintptr_t>(p) & 255u))
       BQ_FAIL(BQ_ERR_HIP, "the static scratch array resolved to %p", p);
+    void* t = nullptr;
+    BQ_HIP(hipGetSymbolAddress(&t, HIP_SYMBOL(static_tickets)));
+    if (t == nullptr || (reinterpret_cast<uintptr_t>(t) & 255u))
+      BQ_FAIL(BQ_ERR_HIP, "the static ticket counters resolved to %p", t);
     ptrs[ordinal] = p;
+    tickets[ordinal] = static_cast<unsigned*>(t);
   }
   *out = ptrs[ordinal];
+  if (tickets_out) *tickets_out = tickets[ordinal];
   return BQ_OK;
 }
 
@@ -966,7 +1012,8 @@ extern "C" bq_status bqk_q_linear_static(const void* x, int32_t x_dtype, size_t 
             "use bqk_q_linear with a workspace",
             need, static_cast<size_t>(BQK_STATIC_SCRATCH_BYTES));
   void* ws = nullptr;
-  BQ_TRY(static_scratch_ptr(&ws));
+  unsigned* tickets = nullptr;
+  BQ_TRY(static_scratch_ptr(&ws, &tickets));
   return q_matmul_core(x, x_dtype, m, k, n, w_values, w_scales, block, value, store, bias, out_dtype, out, ws,
-                       BQK_STATIC_SCRATCH_BYTES, stream);
+                       BQK_STATIC_SCRATCH_BYTES, stream, nullptr, tickets);
 }

@@ -382,6 +382,10 @@ extern "C" bq_status bq_device_open(int32_t ordinal, bq_device** out) {
     }
   }
   hipError_t se = hipStreamCreateWithFlags(&dev->stream, hipStreamNonBlocking);
+  // the ticket counters of the single-launch split-K sum: zero from here on, every launch leaves them so
+  if (se == hipSuccess) se = hipMalloc(reinterpret_cast<void**>(&dev->tickets), kTicketBytes);
+  if (se == hipSuccess) se = hipMemset(dev->tickets, 0, kTicketBytes);
+  if (se == hipSuccess) se = hipDeviceSynchronize();
   if (se == hipSuccess) se = hipEventCreate(&dev->ev_start);
   if (se == hipSuccess) se = hipEventCreate(&dev->ev_stop);
   if (se != hipSuccess) {
@@ -400,6 +404,7 @@ extern "C" bq_status bq_device_close(bq_device* dev) {
   BQ_HIP(hipStreamSynchronize(dev->stream));
   BQ_TRY(dev->trim());
   if (dev->workspace) (void)hipFree(dev->workspace);
+  if (dev->tickets) (void)hipFree(dev->tickets);
   if (dev->validate_cells) (void)hipFree(dev->validate_cells);
   for (int i = 0; i < 2; ++i) {
     if (dev->stage[i]) (void)hipHostFree(dev->stage[i]);
@@ -1279,12 +1284,13 @@ static bq_status q_matmul_impl(const bq_tensor* lhs, const bq_tensor* rhs, int32
     for (size_t b = 0; b < d.batches && rc == BQ_OK; ++b) {
       size_t lb, rb;
       batch_offsets(d, b, &lb, &rb);
-      rc = bqk_q_linear(static_cast<char*>(l->data) + lb * d.m * d.k * dtype_size(lhs_dtype), lhs_dtype,
-                        d.m, d.k, d.n, static_cast<char*>(rhs->data) + rb * vbytes_per_batch,
-                        rhs->scales() + rb * scales_per_batch, static_cast<int32_t>(run), rv,
-                        rhs->scheme.store, bias, out_dtype,
-                        static_cast<char*>(o->data) + b * d.m * d.n * dtype_size(out_dtype), dev->workspace,
-                        dev->workspace_bytes, st);
+      // (the ticket counters are shared like the workspace: only under its lock)
+      rc = q_linear_with_tickets(static_cast<char*>(l->data) + lb * d.m * d.k * dtype_size(lhs_dtype), lhs_dtype,
+                                 d.m, d.k, d.n, static_cast<char*>(rhs->data) + rb * vbytes_per_batch,
+                                 rhs->scales() + rb * scales_per_batch, static_cast<int32_t>(run), rv,
+                                 rhs->scheme.store, bias, out_dtype,
+                                 static_cast<char*>(o->data) + b * d.m * d.n * dtype_size(out_dtype), dev->workspace,
+                                 dev->workspace_bytes, lock.owns_lock() ? dev->tickets : nullptr, st);
     }
     if (lock.owns_lock()) lock.unlock();  // (releasing a tensor takes the same mutex)
     if (lf) bq_tensor_release(lf);         // (stream-ordered: the kernels above were enqueued first)

@@ -2001,6 +2001,48 @@ def test_q_linear_bias_epilogue(dev, value, block, m, k, n):
     assert FloatOps.float_into_data(yb).tobytes() == want.tobytes()
 
 
+@pytest.mark.parametrize("value", [QuantValue.Q8S, QuantValue.Q4S])
+@pytest.mark.parametrize("m,k,n,block", [(1, 4096, 14336, 32), (2, 1024, 2048, 32), (4, 4096, 512, 32), (1, 4096, 256, 32),
+                                          (3, 2048, 1152, 0), (8, 512, 1024, 64), (16, 4096, 14336, 32), (16, 2048, 640, 128),
+                                          (32, 1024, 1536, 32), (5, 8192, 128, 32), (1, 96, 4096, 32), (7, 4096, 2048, 0)])
+def test_single_launch_split_k_is_the_two_launch_sum(dev, value, m, k, n, block):
+    """The handle level runs the decode kernel of one or two rows as one launch (the last workgroup of a
+    column strip adds up the K slices); the kernel level, given a plain workspace, runs the same
+    kernel followed by the reduction kernel, as every larger batch does at both levels. Same partial
+    sums, same summation order: the outputs are
+    equal bit for bit, f32 and bf16, with and without a bias, for few and for many K slices, three
+    times in a row (the ticket counters must come back to zero)."""
+    import ctypes as C
+    from burn_amd import _lib
+    L = _lib.lib()
+    rng = np.random.default_rng(m * 131 + n)
+    w = (rng.standard_normal((k, n)) * 0.02).astype(np.float32)
+    scheme = QuantScheme(value=value) if block == 0 else QuantScheme(value=value).per_block((block,))
+    tw = QTensorOps.quantize_dynamic(FloatOps.float_from_data(w, dev), scheme)
+    cval = VAL[value][0]
+    bias_h = rng.standard_normal(n).astype(np.float32)
+    bias = FloatOps.float_from_data(bias_h, dev)
+    need = L.bqk_q_matmul_workspace(m, k, n, ba.F32, cval)
+    ws = FloatOps.float_empty((max(need, 4) // 4 + 64,), dev)
+    for rep in range(3):
+        x_h = rng.standard_normal((m, k)).astype(np.float32)
+        x = FloatOps.float_from_data(x_h, dev)
+        for out_dtype in (ba.F32, ba.BF16):
+            for b in (None, bias):
+                one = FloatOps.float_into_data(ModuleOps.linear(x, tw, b, out_dtype=out_dtype))
+                out = FloatOps.float_empty((m, n), dev, out_dtype)
+                _lib.check(L.bqk_q_linear(x.data_ptr, ba.F32, m, k, n, tw.data_ptr, tw.scales_ptr, block, cval,
+                                          _lib.STORE_PACKED_U32, b.data_ptr if b is not None else None, out_dtype,
+                                          out.data_ptr, ws.data_ptr, need, dev.stream))
+                two = FloatOps.float_into_data(out)
+                assert one.tobytes() == two.tobytes(), f"rep {rep}, out dtype {out_dtype}, bias {b is not None}"
+    # and the product is right
+    values, scales = QTensorOps.q_into_data(tw).split()
+    q = no.unpack_u32(values.view(np.uint32), w.shape, VAL[value][1])
+    got = FloatOps.float_into_data(QTensorOps.q_matmul(x, tw))
+    matmul_check(got, no.q_matmul_f64(x_h, q, scales, [block] if block else None))
+
+
 def test_q_linear_folds_leading_dims(dev):
     from burn_amd import ModuleOps
     rng = np.random.default_rng(9)
