@@ -35,6 +35,7 @@ SOURCES = [
     ("qmatmul.hip", ["-ffp-contract=off"]),
     ("qskinny.hip", ["-ffp-contract=off"]),
     ("qsplit.hip", ["-ffp-contract=off"]),
+    ("qternary.hip", ["-ffp-contract=off"]),
     ("layout.hip", []),
     # (the GEMM's hand-scheduled stage is one fully unrolled loop of 64 MFMA micro-steps, larger
     # than the default limit for "#pragma unroll")

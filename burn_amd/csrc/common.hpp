@@ -227,6 +227,16 @@ bq_status launch_scale_from_cells(const uint32_t* cells, int value, int scale_dt
 bq_status launch_ternary_matmul(const float* x, const uint32_t* w, const float* scale, size_t m, size_t k, size_t n,
                                 float* out, hipStream_t stream);
 
+// The same product on the bf16 matrix cores, order of the sums given up (qternary.hip): partial products
+// of `slices` K slices to `part`, summed by launch_splitk_reduce.
+bool ternary_mfma_ok(size_t m, size_t k, size_t n);
+size_t ternary_workspace(size_t m, size_t k, size_t n);
+bq_status launch_ternary_mfma(const float* x, const uint32_t* w, const float* scale, size_t m, size_t k, size_t n,
+                              float* part, unsigned* slices_out, hipStream_t stream);
+// out[i] = sum over the slices of part[s][i] (+ bias[i % n]) in a fixed order, to f32 or bf16 (qmatmul.hip).
+bq_status launch_splitk_reduce(const float* part, size_t mn, unsigned slices, const float* bias, size_t n,
+                               int32_t out_dtype, void* out, hipStream_t stream);
+
 // dst[0..n) = value, as a kernel (safe to record into a HIP graph, unlike a memset node).
 bq_status launch_fill_u32(uint32_t* dst, size_t n, uint32_t value, hipStream_t stream);
 

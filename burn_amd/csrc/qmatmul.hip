@@ -710,6 +710,13 @@ static bq_status launch_gemv_reduce(const float* part, size_t mn, unsigned slice
   return BQ_OK;
 }
 
+namespace bq {
+bq_status launch_splitk_reduce(const float* part, size_t mn, unsigned slices, const float* bias, size_t n,
+                               int32_t out_dtype, void* out, hipStream_t stream) {
+  return launch_gemv_reduce(part, mn, slices, bias, n, out_dtype, out, stream);
+}
+}  // namespace bq
+
 // out[r][c] = bias[c], or 0 without a bias: the product over an empty K.
 __global__ void empty_k_kernel(const float* __restrict__ bias, size_t mn, size_t n, int out_dtype,
                                void* __restrict__ out) {

@@ -1222,9 +1222,23 @@ static bq_status q_matmul_impl(const bq_tensor* lhs, const bq_tensor* rhs, int32
       rhs->scheme.level == BQ_LEVEL_TENSOR && lhs->dtype == BQ_F32 && out_dtype == BQ_F32 && rhs->rank == 2 && d.n % 16 == 0) {
     bq_tensor* o = nullptr;
     BQ_TRY(new_float(dev, BQ_F32, d.out_shape, d.rank, &o));
-    bq_status rc = launch_ternary_matmul(static_cast<const float*>(lhs->data), static_cast<const uint32_t*>(rhs->data),
-                                         rhs->scales(), d.m, d.k, d.n, static_cast<float*>(o->data), st);
-    if (rc == BQ_OK && bias != nullptr) rc = launch_add_bias(o->data, BQ_F32, bias, d.m, d.n, st);  // linear: matmul, then + bias
+    bq_status rc = BQ_OK;
+    if (!dev->f32_matmul_exact.load() && ternary_mfma_ok(d.m, d.k, d.n)) {
+      // the same sums on the matrix cores, in another order (a fraction of the time; within 1e-5 of
+      // the largest output). bq_device_set_f32_matmul_exact keeps the reference's order.
+      std::unique_lock<std::mutex> lock(dev->mu);  // the split-K workspace is shared by the calls on this device
+      rc = dev->ensure_workspace(ternary_workspace(d.m, d.k, d.n));
+      unsigned slices = 0;
+      if (rc == BQ_OK)
+        rc = launch_ternary_mfma(static_cast<const float*>(lhs->data), static_cast<const uint32_t*>(rhs->data), rhs->scales(),
+                                 d.m, d.k, d.n, static_cast<float*>(dev->workspace), &slices, st);
+      if (rc == BQ_OK)
+        rc = launch_splitk_reduce(static_cast<const float*>(dev->workspace), d.m * d.n, slices, bias, d.n, BQ_F32, o->data, st);
+    } else {
+      rc = launch_ternary_matmul(static_cast<const float*>(lhs->data), static_cast<const uint32_t*>(rhs->data),
+                                 rhs->scales(), d.m, d.k, d.n, static_cast<float*>(o->data), st);
+      if (rc == BQ_OK && bias != nullptr) rc = launch_add_bias(o->data, BQ_F32, bias, d.m, d.n, st);  // linear: matmul, then + bias
+    }
     if (rc != BQ_OK) {
       bq_tensor_release(o);
       return rc;

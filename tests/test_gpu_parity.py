@@ -1122,9 +1122,19 @@ def test_q2s_quantize_dequantize(dev, block):
         assert (got == q_ref.T).all() and gs.reshape(-1).tobytes() == s_ref.reshape(-1).tobytes()
 
 
-def test_q2s_ternary_matmul_is_the_reference_sum(dev):
-    """f32 activations x per-tensor Q2S weight: the multiply-free path, bit for bit the reference's
-    loop (same order of additions), the reference test's own inputs first."""
+@pytest.fixture
+def exact_matmul(dev):
+    """bq_device_set_f32_matmul_exact for the duration of a test."""
+    dev.set_f32_matmul_exact(True)
+    yield dev
+    dev.set_f32_matmul_exact(False)
+
+
+def test_q2s_ternary_matmul_is_the_reference_sum(exact_matmul):
+    """f32 activations x per-tensor Q2S weight under bq_device_set_f32_matmul_exact: the multiply-free
+    path, bit for bit the reference's loop (same order of additions), the reference test's own inputs
+    first. (Weights whose rows are not whole pairs of packed words take this path by default too.)"""
+    dev = exact_matmul
     a = np.float32([[0.5, -1.2, 0.3, 2.0], [1.0, 0.0, -0.7, 0.4], [-2.0, 1.5, 0.1, -0.3]])
     w = np.zeros((4, 16), np.float32)
     w[:, :3] = [[0.9, -0.2, 0.5], [-0.8, 0.1, 0.7], [0.0, 0.6, -0.4], [0.3, -0.9, 0.2]]   # padded to one packed word
@@ -1166,6 +1176,71 @@ def test_q2s_ternary_matmul_is_the_reference_sum(dev):
     qb, sb = unpack_blob(QTensorOps.q_into_data(twb))
     gotb = FloatOps.float_into_data(QTensorOps.q_matmul(FloatOps.float_from_data(x, dev), twb))
     matmul_check(gotb, no.q_matmul_f64(x, qb, sb, [16]))
+
+
+@pytest.mark.parametrize("m,k,n", [(1, 4096, 14336), (16, 4096, 14336), (1, 257, 64), (7, 512, 1056), (17, 96, 32),
+                                   (33, 1000, 544), (4, 8192, 512), (16, 31, 96), (2, 2048, 4096)])
+def test_q2s_ternary_matmul_on_the_matrix_cores(dev, m, k, n):
+    """The default ternary product: the reference's sums (crates/burn-ndarray/src/ops/qtensor.rs:442-517)
+    in another order, on the bf16 matrix cores with two-term activations. Against the float64 product
+    of the dequantized weight: max-normalised error <= 2e-5 (q_matmul's bound is 1e-2, the reference's
+    ternary test allows 2e-2) and burn's permissive rule on every element; a linear layer's bias; the
+    same bits on a second call; exactly 0 for an all-zero weight; and the reference's inf / NaN pattern
+    (a zero weight skips its activation: no 0 * inf)."""
+    rng = np.random.default_rng(m * 7 + k + n)
+    scheme = QuantScheme(value=QuantValue.Q2S)
+    w = rng.standard_normal((k, n)).astype(np.float32)
+    tw = QTensorOps.quantize_dynamic(FloatOps.float_from_data(w, dev), scheme)
+    q, s = unpack_blob(QTensorOps.q_into_data(tw))
+    assert set(np.unique(q).tolist()) == {-1, 0, 1}
+    gamma = s.reshape(-1)[0]
+    x = rng.standard_normal((m, k)).astype(np.float32)
+    x[rng.random(x.shape) < 0.01] *= 40
+    tx = FloatOps.float_from_data(x, dev)
+    got = FloatOps.float_into_data(QTensorOps.q_matmul(tx, tw))
+    ref = (x.astype(np.float64) @ q.astype(np.float64)) * float(gamma)
+    rel = np.abs(got - ref).max() / np.abs(ref).max()
+    assert rel <= 2e-5, rel
+    matmul_check(got, ref)
+    again = FloatOps.float_into_data(QTensorOps.q_matmul(tx, tw))
+    assert again.tobytes() == got.tobytes()
+    bias = rng.standard_normal(n).astype(np.float32)
+    lin = FloatOps.float_into_data(ModuleOps.linear(tx, tw, FloatOps.float_from_data(bias, dev)))
+    assert lin.tobytes() == (got + bias).astype(np.float32).tobytes()
+    # the reference's order on request: bit for bit its loop, and close to the default
+    dev.set_f32_matmul_exact(True)
+    try:
+        ordered = FloatOps.float_into_data(QTensorOps.q_matmul(tx, tw))
+    finally:
+        dev.set_f32_matmul_exact(False)
+    if m * k * n <= 1 << 24:
+        assert ordered.tobytes() == co.ternary_matmul(x, q, gamma).tobytes()
+    assert np.abs(ordered - got).max() <= 2e-5 * np.abs(ref).max()
+    # an all-zero weight: exactly 0, also under infinite activations
+    tz = QTensorOps.quantize_dynamic(FloatOps.float_from_data(np.zeros((k, n), np.float32), dev), scheme)
+    z = FloatOps.float_into_data(QTensorOps.q_matmul(tx, tz))
+    assert (z == 0).all()
+    # infinite and NaN activations: the pattern of the reference's loop, finite outputs as before
+    xs = x.copy()
+    xs[0, k // 3] = np.inf
+    if m > 1:
+        xs[1, k // 2] = -np.inf
+    if m > 2:
+        xs[2, 0] = np.nan
+    if m > 3:
+        xs[3, 1], xs[3, k - 1] = np.inf, np.inf
+    g = FloatOps.float_into_data(QTensorOps.q_matmul(FloatOps.float_from_data(xs, dev), tw))
+    qf = q.astype(np.float32)
+    hits = lambda mask, sign: (mask.astype(np.float32) @ (qf * sign > 0).astype(np.float32)) > 0   # noqa: E731
+    pinf = hits(np.isposinf(xs), 1) | hits(np.isneginf(xs), -1)      # a +inf contribution reaches the output
+    ninf = hits(np.isposinf(xs), -1) | hits(np.isneginf(xs), 1)
+    nan = hits(np.isnan(xs), 1) | hits(np.isnan(xs), -1) | (pinf & ninf)
+    fin = np.where(np.isfinite(xs), xs, 0.0).astype(np.float64) @ q.astype(np.float64) * float(gamma)
+    assert nan.any() == (m > 2) and pinf.any()
+    assert (np.isnan(g) == nan).all()
+    assert (np.isposinf(g) == (pinf & ~nan)).all() and (np.isneginf(g) == (ninf & ~nan)).all()
+    ok = np.isfinite(g)
+    assert ok[4:].all() and np.abs(g[ok] - fin[ok]).max() <= 2e-5 * np.abs(ref).max()
 
 
 # ------------------------------------------------------------------ full-range values
