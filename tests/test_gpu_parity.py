@@ -1133,7 +1133,7 @@ def exact_matmul(dev):
 def test_q2s_ternary_matmul_is_the_reference_sum(exact_matmul):
     """f32 activations x per-tensor Q2S weight under bq_device_set_f32_matmul_exact: the multiply-free
     path, bit for bit the reference's loop (same order of additions), the reference test's own inputs
-    first. (Weights whose rows are not whole pairs of packed words take this path by default too.)"""
+    first. (Weights whose rows are not whole groups of 4 packed words take this path by default too.)"""
     dev = exact_matmul
     a = np.float32([[0.5, -1.2, 0.3, 2.0], [1.0, 0.0, -0.7, 0.4], [-2.0, 1.5, 0.1, -0.3]])
     w = np.zeros((4, 16), np.float32)
@@ -1178,8 +1178,8 @@ def test_q2s_ternary_matmul_is_the_reference_sum(exact_matmul):
     matmul_check(gotb, no.q_matmul_f64(x, qb, sb, [16]))
 
 
-@pytest.mark.parametrize("m,k,n", [(1, 4096, 14336), (16, 4096, 14336), (1, 257, 64), (7, 512, 1056), (17, 96, 32),
-                                   (33, 1000, 544), (4, 8192, 512), (16, 31, 96), (2, 2048, 4096)])
+@pytest.mark.parametrize("m,k,n", [(1, 4096, 14336), (16, 4096, 14336), (1, 257, 64), (7, 512, 1088), (17, 96, 128),
+                                   (33, 1000, 576), (4, 8192, 512), (16, 31, 192), (2, 2048, 4096), (3, 130, 32)])
 def test_q2s_ternary_matmul_on_the_matrix_cores(dev, m, k, n):
     """The default ternary product: the reference's sums (crates/burn-ndarray/src/ops/qtensor.rs:442-517)
     in another order, on the bf16 matrix cores with two-term activations. Against the float64 product
@@ -1190,9 +1190,10 @@ def test_q2s_ternary_matmul_on_the_matrix_cores(dev, m, k, n):
     rng = np.random.default_rng(m * 7 + k + n)
     scheme = QuantScheme(value=QuantValue.Q2S)
     w = rng.standard_normal((k, n)).astype(np.float32)
-    tw = QTensorOps.quantize_dynamic(FloatOps.float_from_data(w, dev), scheme)
+    # (weights as the Quantizer makes them under Calibration::AbsMean: about a third each of -1, 0, +1)
+    tw = QTensorOps.quantize_abs_mean(FloatOps.float_from_data(w, dev), scheme)
     q, s = unpack_blob(QTensorOps.q_into_data(tw))
-    assert set(np.unique(q).tolist()) == {-1, 0, 1}
+    assert set(np.unique(q).tolist()) == {-1, 0, 1} and (q != 0).mean() > 0.4
     gamma = s.reshape(-1)[0]
     x = rng.standard_normal((m, k)).astype(np.float32)
     x[rng.random(x.shape) < 0.01] *= 40
