@@ -1260,7 +1260,10 @@ static bq_status q_matmul_impl(const bq_tensor* lhs, const bq_tensor* rhs, int32
   }
   if (fused && (d.n % static_cast<size_t>(num_quants(rv)))) fused = false;
   // (f32 activations, more than 32 rows: the fast kernels round to bf16; the device may ask for f32)
-  if (fused && lhs_dtype == BQ_F32 && d.m > 32 && dev->f32_matmul_exact.load()) fused = false;
+  // (more than 32 rows: the fast kernel rounds s * q -- and f32 activations -- to bf16; the device may ask
+  // for the reference's arithmetic instead: weights dequantized to f32, f32 products)
+  const bool exact = !lq && d.m > 32 && dev->f32_matmul_exact.load();
+  if (fused && exact) fused = false;
   if (fused && !fused_matmul_ok(d.m, d.k, d.n, lhs_dtype, rv,
                                 run > 0 ? d.n / static_cast<size_t>(run) : 0))
     fused = false;
@@ -1321,7 +1324,9 @@ static bq_status q_matmul_impl(const bq_tensor* lhs, const bq_tensor* rhs, int32
   bq_tensor* rf = nullptr;
   bq_status rc = BQ_OK;
   if (lq) rc = bq_dequantize(lhs, target, &lf);
-  if (rc == BQ_OK && rq) rc = bq_dequantize(rhs, target, &rf);
+  // (exact mode with bf16 activations: the weights still go to f32 -- dequantized to bf16, as the
+  // reference's dtype rule has it, they would be rounded exactly as the fast kernel rounds them)
+  if (rc == BQ_OK && rq) rc = bq_dequantize(rhs, exact ? BQ_F32 : target, &rf);
   bq_tensor* o = nullptr;
   if (rc == BQ_OK) rc = new_float(dev, out_dtype, d.out_shape, d.rank, &o);
   if (rc == BQ_OK) {
@@ -1369,12 +1374,24 @@ extern "C" bq_status bq_q_matmul_propagate(const bq_tensor* lhs, const bq_tensor
   const bool lq = lhs->dtype == BQ_QFLOAT, rq = rhs->dtype == BQ_QFLOAT;
   if (!lq && !rq) BQ_FAIL(BQ_ERR_DTYPE, "q_matmul needs at least one quantized operand");
   const int32_t target = !lq ? lhs->dtype : (!rq ? rhs->dtype : BQ_F32);
-  if (target != BQ_F32)
-    BQ_FAIL(BQ_ERR_UNSUPPORTED_OP, "q_matmul with propagation quantizes an f32 product; the float operand is bf16");
   const bq_scheme scheme = rq ? rhs->scheme : lhs->scheme;
+  // The product has the float operand's dtype (qtensor.rs:234-239). A bf16 product is what gets
+  // quantized: its values, widened exactly to the f32 the quantize kernels read.
   bq_tensor* f = nullptr;
-  BQ_TRY(q_matmul_impl(lhs, rhs, BQ_F32, nullptr, &f));
-  bq_status rc = bq_quantize_dynamic(f, &scheme, out);
+  BQ_TRY(q_matmul_impl(lhs, rhs, target, nullptr, &f));
+  bq_status rc = BQ_OK;
+  if (target == BQ_BF16) {
+    bq_tensor* wide = nullptr;
+    rc = new_float(f->dev, BQ_F32, f->shape, f->rank, &wide);
+    if (rc == BQ_OK) rc = launch_bf16_to_f32(static_cast<const uint16_t*>(f->data), f->numel(), static_cast<float*>(wide->data), f->dev->stream);
+    bq_tensor_release(f);
+    f = wide;
+    if (rc != BQ_OK) {
+      if (f) bq_tensor_release(f);
+      return rc;
+    }
+  }
+  rc = bq_quantize_dynamic(f, &scheme, out);
   bq_tensor_release(f);
   return rc;
 }

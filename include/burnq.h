@@ -119,13 +119,16 @@ bq_status bq_device_trim(bq_device* dev);
  * stream (a debugging aid; refused during graph capture). Off, such inputs give unspecified
  * integers. */
 bq_status bq_device_set_validate(bq_device* dev, int32_t on);
-/* f32 activations against a quantized weight keep at least 16 significant bits per product up to
- * 32 rows; from 33 rows on the fast kernel rounds them (and s * q) to bf16, about 2e-3 of the
+/* Activations against a quantized weight keep at least 16 significant bits per product up to 32
+ * rows; from 33 rows on the fast kernel multiplies bf16(activation) by bf16(s * q), about 2e-3 of the
  * largest output, inside the 1e-2 the reference's own tests allow
  * (crates/burn-backend-tests/tests/tensor/float/quantization/ops/matmul.rs) but far from its f32
- * sgemm. on != 0 makes q_matmul / q_linear on this device multiply such products the reference's
- * way instead -- dequantize to f32, f32 matrix product -- at a fraction of the speed. Off by
- * default. No counterpart in the reference. */
+ * sgemm: on a 4096-deep product a few outputs in a million leave burn's elementwise rule
+ * (|y - y'| < max(1e-2 max(|y|, |y'|), 1e-2)). on != 0 makes q_matmul / q_linear on this device
+ * multiply such products the reference's way instead -- weights dequantized to f32, f32 matrix
+ * product, for f32 and bf16 activations alike -- at a fraction of the speed, and makes the ternary
+ * product (Q2S weights) keep the reference's order of additions bit for bit instead of running on
+ * the matrix cores. Off by default. No counterpart in the reference. */
 bq_status bq_device_set_f32_matmul_exact(bq_device* dev, int32_t on);
 /* HIP-event stopwatch on the context's stream (what Backend::sync-bracketed benches measure,
  * without the host round trip): start, enqueue work, stop -> elapsed milliseconds. */
@@ -253,8 +256,8 @@ bq_status bq_q_matmul_as(const bq_tensor* lhs, const bq_tensor* rhs, int32_t out
 /* q_matmul under QuantPropagation::Propagate (burn-ndarray/src/ops/qtensor.rs:262-265; the setting
  * is crates/burn-std/src/tensor/quantization.rs:28-75): the float product is quantized again,
  * quantize_dynamic with the scheme of the quantized operand (the rhs's when both are), and a
- * quantized tensor is returned. The product is f32; a bf16 float operand returns
- * BQ_ERR_UNSUPPORTED_OP. */
+ * quantized tensor is returned. The product has the float operand's dtype, as there: with a bf16
+ * operand it is the bf16 product whose values are quantized. */
 bq_status bq_q_matmul_propagate(const bq_tensor* lhs, const bq_tensor* rhs, bq_tensor** out);
 /* linear with a quantized weight (crates/burn-tensor/src/tensor/module.rs:527-567, what
  * nn::Linear::forward reaches after Module::quantize_weights,

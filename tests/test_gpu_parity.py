@@ -549,6 +549,36 @@ def test_f32_matmul_exact_setting_removes_the_step_at_33_rows(dev, value):
     assert small <= 2e-5 and small == rel(QTensorOps.q_matmul(FloatOps.float_from_data(x[:32], dev), tq), ref[:32])
 
 
+def test_matmul_exact_setting_with_bf16_activations(dev):
+    """bf16 activations x Q4S block-32, K = 4096 (the prefill configuration's depth, a quarter of its
+    width): the fast kernel rounds s * q to bf16, which on a product this deep puts a few outputs in a
+    million outside burn's elementwise rule; with the setting on the weights are dequantized to f32 and
+    multiplied in f32, and every output meets the rule -- f32 and bf16 output, with a bias."""
+    rng = np.random.default_rng(55)
+    m, k, n = 2048, 4096, 3584
+    w = (rng.standard_normal((k, n)) * 0.02).astype(np.float32)
+    tq = QTensorOps.quantize_dynamic(FloatOps.float_from_data(w, dev), QuantScheme(value=QuantValue.Q4S).per_block((32,)))
+    q, s = unpack_blob(QTensorOps.q_into_data(tq))
+    bits = ba.bf16_bits_from_f32(rng.standard_normal((m, k)).astype(np.float32))
+    x = ba.f32_from_bf16_bits(bits)
+    xt = FloatOps.float_from_data(bits, dev, ba.BF16)
+    ref = no.q_matmul_f64(x, q, s, [32])
+    fast = FloatOps.float_into_data(QTensorOps.q_matmul(xt, tq, out_dtype=ba.F32))
+    outside_fast = int((~burn_approx_eq(fast, ref, 1e-2, 1e-2)).sum())
+    assert np.abs(fast - ref).max() / np.abs(ref).max() <= 1e-2
+    dev.set_f32_matmul_exact(True)
+    try:
+        exact = FloatOps.float_into_data(QTensorOps.q_matmul(xt, tq, out_dtype=ba.F32))
+        bias = rng.standard_normal(n).astype(np.float32)
+        lin = FloatOps.float_into_data(ModuleOps.linear(xt, tq, FloatOps.float_from_data(bias, dev), out_dtype=ba.F32))
+    finally:
+        dev.set_f32_matmul_exact(False)
+    assert np.abs(exact - ref).max() / np.abs(ref).max() <= 1e-5      # f32 sums over 4096 terms
+    assert burn_approx_eq(exact, ref, 1e-2, 1e-2).all()
+    assert burn_approx_eq(lin, ref + bias[None, :].astype(np.float64), 1e-2, 1e-2).all()
+    assert outside_fast <= 30, outside_fast       # (7.3 M outputs at 4.7 sigma: about 19 predicted)
+
+
 def test_host_transfers_around_the_staging_size(dev):
     """Host buffers travel through two pinned halves of 2 MiB: sizes just under, at and over one and
     two halves, and far over, come back byte for byte, for float tensors and for quantized blobs
@@ -2161,8 +2191,13 @@ def test_q_matmul_propagate_requantizes(dev, value, block):
     q_ref, s_ref = co.quantize_dynamic(prod, oscheme(scheme))
     q, s = unpack_blob(QTensorOps.q_into_data(out))
     assert (q == q_ref).all() and s.tobytes() == s_ref.tobytes()
-    with pytest.raises(ba.BurnqError):
-        QTensorOps.q_matmul_propagate(FloatOps.float_from_data(ba.bf16_bits_from_f32(x), dev, ba.BF16), tq)
+    # a bf16 operand: the product is bf16 (the float operand's dtype), and its values are what is quantized
+    tb = FloatOps.float_from_data(ba.bf16_bits_from_f32(x), dev, ba.BF16)
+    out_b = QTensorOps.q_matmul_propagate(tb, tq)
+    prod_b = ba.f32_from_bf16_bits(FloatOps.float_into_data(QTensorOps.q_matmul(tb, tq)))
+    q_ref, s_ref = co.quantize_dynamic(prod_b, oscheme(scheme))
+    q, s = unpack_blob(QTensorOps.q_into_data(out_b))
+    assert out_b.is_quantized and (q == q_ref).all() and s.tobytes() == s_ref.tobytes()
 
 
 def test_q_matmul_empty_k_is_zero(dev):
