@@ -84,14 +84,63 @@ def graph_ms(dev, fn, count, steps, warmup):
     return ev / count
 
 
+_GAMMA = np.uint64(0x9E3779B97F4A7C15)
+
+
+def _splitmix64_mix(z):
+    """The output function of splitmix64 on an array of states (uint64, wrapping arithmetic)."""
+    z = (z ^ (z >> np.uint64(30))) * np.uint64(0xBF58476D1CE4E5B9)
+    z = (z ^ (z >> np.uint64(27))) * np.uint64(0x94D049BB133111EB)
+    return z ^ (z >> np.uint64(31))
+
+
+_INPUT_CACHE = {}
+
+
 def normal_f32(seed, shape, scale=1.0, outliers=False):
-    rng = np.random.default_rng(seed)
-    x = rng.standard_normal(shape, dtype=np.float32)
-    if scale != 1.0:
-        x *= np.float32(scale)
-    if outliers:
-        x[rng.random(shape, dtype=np.float32) < 0.01] *= 50
-    return x
+    """Cached (read-only) wrapper of generate_normal_f32: the same big tensor feeds several legs."""
+    key = (seed, tuple(shape), scale, outliers)
+    if key not in _INPUT_CACHE:
+        x = generate_normal_f32(seed, shape, scale, outliers)
+        x.setflags(write=False)
+        if x.size < (1 << 20):
+            return x
+        _INPUT_CACHE[key] = x
+    return _INPUT_CACHE[key]
+
+
+def generate_normal_f32(seed, shape, scale=1.0, outliers=False):
+    """Deterministic inputs of the measurement spec: the splitmix64 stream seeded with `seed`
+    (state_i = seed + (i + 1) * 0x9E3779B97F4A7C15, output mix(state_i)) -> Box-Muller in float64
+    (outputs 2j and 2j + 1 give elements 2j and 2j + 1) -> float32. outliers: element i is scaled by
+    50 iff splitmix64(seed ^ i) % 100 == 0 (the first output of a generator seeded with seed ^ i).
+    Generated in chunks; the same bytes on every machine up to libm's log / sin / cos."""
+    n = int(np.prod(shape))
+    out = np.empty(n, np.float32)
+    chunk = 1 << 22
+    with np.errstate(over="ignore"):
+        for lo in range(0, n, chunk):
+            hi = min(n, lo + chunk)
+            first = lo - (lo & 1)                                  # whole Box-Muller pairs
+            count = (hi - first + 1) // 2 * 2
+            idx = np.arange(first, first + count, dtype=np.uint64)
+            z = _splitmix64_mix(np.uint64(seed) + (idx + np.uint64(1)) * _GAMMA)
+            u = (z >> np.uint64(11)).astype(np.float64) * (1.0 / 9007199254740992.0)   # [0, 1)
+            r = np.sqrt(-2.0 * np.log(1.0 - u[0::2]))             # 1 - u in (0, 1]
+            theta = (2.0 * np.pi) * u[1::2]
+            pair = np.empty(count, np.float64)
+            pair[0::2] = r * np.cos(theta)
+            pair[1::2] = r * np.sin(theta)
+            vals = pair[lo - first:hi - first]
+            if scale != 1.0:
+                vals = vals * scale
+            vals = vals.astype(np.float32)
+            if outliers:
+                i = np.arange(lo, hi, dtype=np.uint64)
+                pick = _splitmix64_mix((np.uint64(seed) ^ i) + _GAMMA) % np.uint64(100) == 0
+                vals[pick] *= np.float32(50)
+            out[lo:hi] = vals
+    return out.reshape(shape)
 
 
 def roofline(bound, achieved, peak, unit, kernel, avg_launch_ms):
