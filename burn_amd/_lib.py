@@ -18,7 +18,7 @@ OK, ERR_NULL, ERR_UNSUPPORTED_SCHEME, ERR_SHAPE, ERR_DTYPE, ERR_HIP, ERR_SIZE, E
 STATUS_NAMES = ["OK", "ERR_NULL", "ERR_UNSUPPORTED_SCHEME", "ERR_SHAPE", "ERR_DTYPE", "ERR_HIP",
                 "ERR_SIZE", "ERR_UNSUPPORTED_OP", "ERR_NONFINITE"]
 # dtypes
-F32, BF16, QFLOAT = 0, 1, 2
+F32, BF16, QFLOAT, I32, I64 = 0, 1, 2, 3, 4
 # scheme enums
 Q8S, Q4S, Q2S, Q8F, Q4F, Q2F = 0, 1, 2, 3, 4, 5
 LEVEL_TENSOR, LEVEL_BLOCK = 0, 1
@@ -118,6 +118,14 @@ SIGNATURES = {
     "bq_q_swap_dims": (_i32, [_vp, _i32, _i32, _pvp]),
     "bq_q_permute": (_i32, [_vp, C.POINTER(_i32), _i32, _pvp]),
     "bq_q_flip": (_i32, [_vp, C.POINTER(_i32), _i32, _pvp]),
+    "bq_int_from_data": (_i32, [_vp, _vp, _i32, _psz, _i32, _pvp]),
+    "bq_int_into_data": (_i32, [_vp, _vp, _sz]),
+    "bq_q_slice": (_i32, [_vp, C.POINTER(C.c_int64), C.POINTER(C.c_int64), C.POINTER(C.c_int64), _i32, _pvp]),
+    "bq_q_select": (_i32, [_vp, _i32, _vp, _pvp]),
+    "bq_q_gather": (_i32, [_i32, _vp, _vp, _pvp]),
+    "bq_q_expand": (_i32, [_vp, _psz, _i32, _pvp]),
+    "bq_q_argmax": (_i32, [_vp, _i32, _i32, _pvp]),
+    "bq_q_argmin": (_i32, [_vp, _i32, _i32, _pvp]),
     "bqk_selftest_division": (_i32, [_vp, _vp]),
     "bqk_copy": (_i32, [_vp, _vp, _sz, _vp]),
     "bqk_lds_request_status": (_i32, [_sz, _sz]),

@@ -204,6 +204,17 @@ bq_status launch_q_gather(const void* src, void* dst, const size_t* src_shape, i
                           const uint8_t* flip, int value, bool native, hipStream_t stream);
 bq_status launch_f32_gather(const float* src, float* dst, const size_t* src_shape, int rank, const int32_t* axes,
                             const uint8_t* flip, hipStream_t stream);
+// Integer-domain slice / select / gather / expand (layout.hip): output element e with coordinates c reads
+// source element base + sum_a c[a] * stride[a], the coordinate of index_dim replaced by
+// indices[c[index_dim]] (index_mode 1) or indices[e] (index_mode 2), clamped into [0, index_limit).
+bq_status launch_q_index_map(const void* src, void* dst, const size_t* out_shape, int rank, const int64_t* stride, int64_t base,
+                             int index_dim, int index_mode, const void* indices, int index_dtype, size_t index_limit, int value,
+                             bool src_native, bool dst_native, hipStream_t stream);
+bq_status launch_f32_index_map(const float* src, float* dst, const size_t* out_shape, int rank, const int64_t* stride, int64_t base,
+                               int index_dim, int index_mode, const void* indices, int index_dtype, size_t index_limit,
+                               hipStream_t stream);
+bq_status launch_q_arg(const void* src, int value, bool native, size_t outer, size_t len, size_t inner, bool want_max, int out_dtype,
+                       void* out, hipStream_t stream);
 // out[r][c] += bias[c] (out f32 or bf16, in place), and a bf16 -> f32 copy (qmatmul.hip).
 bq_status launch_add_bias(void* out, int out_dtype, const float* bias, size_t m, size_t n, hipStream_t stream);
 bq_status launch_bf16_to_f32(const uint16_t* src, size_t n, float* dst, hipStream_t stream);

@@ -1,5 +1,7 @@
 // Layout ops on quantized tensors for gfx950: q_permute / q_swap_dims / q_flip
-// (crates/burn-ndarray/src/ops/qtensor.rs:301-347). The reference permutes the values and, for
+// (crates/burn-ndarray/src/ops/qtensor.rs:301-347), and the ops the reference's CPU backend runs on
+// the integers without dequantizing (same file, :349-430): q_slice, q_select, q_gather, q_expand,
+// q_argmax, q_argmin (the index map and arg kernels at the end of this file). The reference permutes the values and, for
 // block schemes, the scales with their blocks (scheme.permute_block_dims); tensors here are
 // always dense row-major, so the result is materialised: by a tiled transpose when 8-bit values
 // swap their last two dims (a transposed weight, the usual case), else by a gather, one thread per
@@ -205,6 +207,174 @@ bq_status launch_f32_gather(const float* src, float* dst, const size_t* src_shap
     hipLaunchKernelGGL(f32_gather_kernel<uint32_t>, dim3(static_cast<unsigned>((n + 255) / 256)), dim3(256), 0, st, src, dst, n, d);
   else
     hipLaunchKernelGGL(f32_gather_kernel<size_t>, dim3(static_cast<unsigned>((n + 255) / 256)), dim3(256), 0, st, src, dst, n, d);
+  BQ_HIP(hipGetLastError());
+  return BQ_OK;
+}
+
+// ---- integer-domain slice / select / gather / expand ---------------------------------------------
+// One kernel for all four: output element e with coordinates c reads source element
+//   base + sum over dims a != index_dim of c[a] * stride[a] + i * stride[index_dim],
+// i = c[index_dim] (slice, expand: a negative stride runs backwards, a zero stride broadcasts),
+// indices[c[index_dim]] (select) or indices[e] (gather). An index outside its dim, which the
+// reference panics on, is clamped into it: never a fault.
+namespace {
+
+struct IndexMap {
+  int rank;
+  uint32_t shape[BQ_MAX_RANK];   // output shape
+  int64_t stride[BQ_MAX_RANK];   // source elements per step of output dim a
+  int64_t base;
+  int index_dim;                 // -1: none
+  int index_mode;                // 1: indices[c[index_dim]] (select), 2: indices[e] (gather)
+  int index_i64;                 // indices are i64 (else i32)
+  int64_t index_limit;           // extent of the source dim the indices address
+};
+
+__device__ __forceinline__ int64_t mapped_index(const IndexMap& d, size_t e, const void* __restrict__ indices) {
+  int64_t idx = d.base;
+  size_t rem = e;
+  for (int a = d.rank - 1; a >= 0; --a) {
+    const size_t c = rem % d.shape[a];
+    rem /= d.shape[a];
+    int64_t i = static_cast<int64_t>(c);
+    if (a == d.index_dim) {
+      const size_t at = d.index_mode == 2 ? e : c;
+      i = d.index_i64 ? static_cast<const int64_t*>(indices)[at] : static_cast<int64_t>(static_cast<const int32_t*>(indices)[at]);
+      i = i < 0 ? 0 : (i >= d.index_limit ? d.index_limit - 1 : i);
+    }
+    idx += i * d.stride[a];
+  }
+  return idx;
+}
+
+template <int BITS>
+__global__ void __launch_bounds__(256)
+q_index_map_kernel(const uint32_t* __restrict__ src, uint32_t* __restrict__ dst, size_t n, IndexMap d, bool src_native, bool dst_native,
+                   const void* __restrict__ indices) {
+  constexpr int EPW = 32 / BITS;
+  const size_t unit = static_cast<size_t>(blockIdx.x) * 256 + threadIdx.x;
+  const size_t e0 = unit * EPW;
+  if (e0 >= n) return;
+  uint32_t word = 0;
+#pragma unroll
+  for (int j = 0; j < EPW; ++j) {
+    const size_t e = e0 + j;
+    if (e >= n) break;
+    const size_t idx = static_cast<size_t>(mapped_index(d, e, indices));
+    uint32_t v;
+    if (BITS == 8 || src_native)
+      v = reinterpret_cast<const uint8_t*>(src)[idx] & ((1u << BITS) - 1u);
+    else  // (rows are whole words, so flat element idx sits in word idx / EPW)
+      v = (src[idx / EPW] >> (BITS * (idx % EPW))) & ((1u << BITS) - 1u);
+    word |= v << (BITS * j);
+  }
+  if (!dst_native) {
+    dst[unit] = word;
+  } else {  // one i8 per value: sign-extend the field
+    for (int j = 0; j < EPW && e0 + j < n; ++j)
+      reinterpret_cast<int8_t*>(dst)[e0 + j] = static_cast<int8_t>(static_cast<int32_t>(word << (32 - BITS * (j + 1))) >> (32 - BITS));
+  }
+}
+
+__global__ void __launch_bounds__(256)
+f32_index_map_kernel(const float* __restrict__ src, float* __restrict__ dst, size_t n, IndexMap d, const void* __restrict__ indices) {
+  const size_t e = static_cast<size_t>(blockIdx.x) * 256 + threadIdx.x;
+  if (e < n) dst[e] = src[mapped_index(d, e, indices)];
+}
+
+// q_argmax / q_argmin on the stored integers: per output position, the first index along `dim` of the
+// largest (smallest) value -- ties keep the lowest index, as the reference's fold with a strict
+// comparison does (crates/burn-ndarray/src/ops/base.rs:1727-1750). One thread per output position.
+template <int BITS>
+__global__ void __launch_bounds__(256)
+q_arg_kernel(const uint32_t* __restrict__ src, bool native, size_t outer, size_t len, size_t inner, bool want_max, bool out_i64,
+             void* __restrict__ out) {
+  constexpr int EPW = 32 / BITS;
+  const size_t pos = static_cast<size_t>(blockIdx.x) * 256 + threadIdx.x;
+  if (pos >= outer * inner) return;
+  const size_t o = pos / inner, in = pos % inner;
+  int best = 0;
+  size_t best_at = 0;
+  for (size_t i = 0; i < len; ++i) {
+    const size_t idx = (o * len + i) * inner + in;
+    int v;
+    if (BITS == 8 || native) v = reinterpret_cast<const int8_t*>(src)[idx];
+    else v = static_cast<int32_t>(src[idx / EPW] << (32 - BITS - BITS * (idx % EPW))) >> (32 - BITS);
+    if (i == 0 || (want_max ? v > best : v < best)) {
+      best = v;
+      best_at = i;
+    }
+  }
+  if (out_i64) static_cast<int64_t*>(out)[pos] = static_cast<int64_t>(best_at);
+  else static_cast<int32_t*>(out)[pos] = static_cast<int32_t>(best_at);
+}
+
+IndexMap make_index_map(const size_t* out_shape, int rank, const int64_t* stride, int64_t base, int index_dim, int index_mode,
+                        int index_dtype, size_t index_limit) {
+  IndexMap d{};
+  d.rank = rank;
+  for (int a = 0; a < rank; ++a) {
+    d.shape[a] = static_cast<uint32_t>(out_shape[a]);
+    d.stride[a] = stride[a];
+  }
+  d.base = base;
+  d.index_dim = index_dim;
+  d.index_mode = index_mode;
+  d.index_i64 = index_dtype == BQ_I64;
+  d.index_limit = static_cast<int64_t>(index_limit);
+  return d;
+}
+
+}  // namespace
+
+// Values of `out_shape` (every extent below 2^32) gathered through the index map described above.
+// `indices` (device memory, BQ_I32 or BQ_I64) is read when index_dim >= 0.
+bq_status launch_q_index_map(const void* src, void* dst, const size_t* out_shape, int rank, const int64_t* stride, int64_t base,
+                             int index_dim, int index_mode, const void* indices, int index_dtype, size_t index_limit, int value,
+                             bool src_native, bool dst_native, hipStream_t st) {
+  size_t n = 1;
+  for (int a = 0; a < rank; ++a) n *= out_shape[a];
+  if (n == 0) return BQ_OK;
+  const IndexMap d = make_index_map(out_shape, rank, stride, base, index_dim, index_mode, index_dtype, index_limit);
+  const int bits = value_bits(value);
+  const size_t units = (n + 32 / bits - 1) / (32 / bits);
+  if ((units + 255) / 256 > 0x7FFFFFFFu) BQ_FAIL(BQ_ERR_SIZE, "an index map over %zu values exceeds the launch grid", n);
+  dim3 grid(static_cast<unsigned>((units + 255) / 256)), tb(256);
+  const uint32_t* s32 = static_cast<const uint32_t*>(src);
+  uint32_t* d32 = static_cast<uint32_t*>(dst);
+  if (bits == 8) hipLaunchKernelGGL(q_index_map_kernel<8>, grid, tb, 0, st, s32, d32, n, d, src_native, dst_native, indices);
+  else if (bits == 4) hipLaunchKernelGGL(q_index_map_kernel<4>, grid, tb, 0, st, s32, d32, n, d, src_native, dst_native, indices);
+  else hipLaunchKernelGGL(q_index_map_kernel<2>, grid, tb, 0, st, s32, d32, n, d, src_native, dst_native, indices);
+  BQ_HIP(hipGetLastError());
+  return BQ_OK;
+}
+
+// The same for an f32 tensor (the block scales, in params_shape order).
+bq_status launch_f32_index_map(const float* src, float* dst, const size_t* out_shape, int rank, const int64_t* stride, int64_t base,
+                               int index_dim, int index_mode, const void* indices, int index_dtype, size_t index_limit, hipStream_t st) {
+  size_t n = 1;
+  for (int a = 0; a < rank; ++a) n *= out_shape[a];
+  if (n == 0) return BQ_OK;
+  const IndexMap d = make_index_map(out_shape, rank, stride, base, index_dim, index_mode, index_dtype, index_limit);
+  if ((n + 255) / 256 > 0x7FFFFFFFu) BQ_FAIL(BQ_ERR_SIZE, "an index map over %zu scales exceeds the launch grid", n);
+  hipLaunchKernelGGL(f32_index_map_kernel, dim3(static_cast<unsigned>((n + 255) / 256)), dim3(256), 0, st, src, dst, n, d, indices);
+  BQ_HIP(hipGetLastError());
+  return BQ_OK;
+}
+
+// out[outer][1][inner] = arg max / min over the `len` values along the reduced dim (i32 or i64).
+bq_status launch_q_arg(const void* src, int value, bool native, size_t outer, size_t len, size_t inner, bool want_max, int out_dtype,
+                       void* out, hipStream_t st) {
+  const size_t n = outer * inner;
+  if (n == 0) return BQ_OK;
+  if ((n + 255) / 256 > 0x7FFFFFFFu) BQ_FAIL(BQ_ERR_SIZE, "an arg reduction over %zu positions exceeds the launch grid", n);
+  dim3 grid(static_cast<unsigned>((n + 255) / 256)), tb(256);
+  const uint32_t* s32 = static_cast<const uint32_t*>(src);
+  const int bits = value_bits(value);
+  const bool i64 = out_dtype == BQ_I64;
+  if (bits == 8) hipLaunchKernelGGL(q_arg_kernel<8>, grid, tb, 0, st, s32, native, outer, len, inner, want_max, i64, out);
+  else if (bits == 4) hipLaunchKernelGGL(q_arg_kernel<4>, grid, tb, 0, st, s32, native, outer, len, inner, want_max, i64, out);
+  else hipLaunchKernelGGL(q_arg_kernel<2>, grid, tb, 0, st, s32, native, outer, len, inner, want_max, i64, out);
   BQ_HIP(hipGetLastError());
   return BQ_OK;
 }

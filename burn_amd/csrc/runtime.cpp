@@ -2,6 +2,7 @@
 // wire format and the QTensorOps entry points (validation + kernel dispatch). No arithmetic on
 // tensor contents happens on the host: every value is produced by a HIP kernel.
 #include <algorithm>
+#include <cstdint>
 #include <cstring>
 
 #include "common.hpp"
@@ -532,11 +533,12 @@ extern "C" bq_status bq_graph_release(bq_graph* g) {
 }
 
 // ================================================================================ handles
-static size_t dtype_size(int32_t dtype) { return dtype == BQ_BF16 ? 2 : 4; }
+static size_t dtype_size(int32_t dtype) { return dtype == BQ_BF16 ? 2 : (dtype == BQ_I64 ? 8 : 4); }
 
 static bq_status new_float(bq_device* dev, int32_t dtype, const size_t* shape, int32_t rank,
                            bq_tensor** out) {
-  if (dtype != BQ_F32 && dtype != BQ_BF16) BQ_FAIL(BQ_ERR_DTYPE, "float dtype must be f32 or bf16");
+  // (the same dense row-major layout carries the i32 / i64 index tensors of q_select, q_gather, q_argmax)
+  if (dtype != BQ_F32 && dtype != BQ_BF16 && dtype != BQ_I32 && dtype != BQ_I64) BQ_FAIL(BQ_ERR_DTYPE, "dtype must be f32, bf16, i32 or i64");
   if (rank < 1 || rank > BQ_MAX_RANK) BQ_FAIL(BQ_ERR_SHAPE, "rank %d outside 1..%d", rank, BQ_MAX_RANK);
   BQ_TRY(check_shape_size(shape, rank));
   bq_tensor* t = new bq_tensor();
@@ -627,14 +629,35 @@ extern "C" size_t bq_tensor_num_scales(const bq_tensor* t) { return t ? t->num_s
 // ================================================================================ float tensors
 extern "C" bq_status bq_float_empty(bq_device* dev, int32_t dtype, const size_t* shape, int32_t rank,
                                     bq_tensor** out) {
+  if (dtype != BQ_F32 && dtype != BQ_BF16) BQ_FAIL(BQ_ERR_DTYPE, "float dtype must be f32 or bf16");
   BQ_NOTNULL(dev);
   BQ_NOTNULL(shape);
   BQ_NOTNULL(out);
   return new_float(dev, dtype, shape, rank, out);
 }
 
+static bq_status plain_from_data(bq_device* dev, const void* host, int32_t dtype, const size_t* shape, int32_t rank, bq_tensor** out);
+
 extern "C" bq_status bq_float_from_data(bq_device* dev, const void* host, int32_t dtype,
                                         const size_t* shape, int32_t rank, bq_tensor** out) {
+  if (dtype != BQ_F32 && dtype != BQ_BF16) BQ_FAIL(BQ_ERR_DTYPE, "float dtype must be f32 or bf16");
+  return plain_from_data(dev, host, dtype, shape, rank, out);
+}
+
+// IntTensorOps::int_from_data / int_into_data for the index tensors the quantized ops take and return.
+extern "C" bq_status bq_int_from_data(bq_device* dev, const void* host, int32_t dtype, const size_t* shape, int32_t rank,
+                                      bq_tensor** out) {
+  if (dtype != BQ_I32 && dtype != BQ_I64) BQ_FAIL(BQ_ERR_DTYPE, "int dtype must be i32 or i64");
+  return plain_from_data(dev, host, dtype, shape, rank, out);
+}
+
+extern "C" bq_status bq_int_into_data(const bq_tensor* t, void* host, size_t capacity_bytes) {
+  BQ_NOTNULL(t);
+  if (t->dtype != BQ_I32 && t->dtype != BQ_I64) BQ_FAIL(BQ_ERR_DTYPE, "bq_int_into_data takes an i32 or i64 tensor");
+  return bq_float_into_data(t, host, capacity_bytes);
+}
+
+static bq_status plain_from_data(bq_device* dev, const void* host, int32_t dtype, const size_t* shape, int32_t rank, bq_tensor** out) {
   BQ_NOTNULL(dev);
   BQ_NOTNULL(shape);
   BQ_NOTNULL(out);
@@ -1174,7 +1197,8 @@ extern "C" bq_status bq_float_matmul(const bq_tensor* lhs, const bq_tensor* rhs,
   BQ_NOTNULL(lhs);
   BQ_NOTNULL(rhs);
   BQ_NOTNULL(out);
-  if (lhs->dtype == BQ_QFLOAT || rhs->dtype == BQ_QFLOAT) BQ_FAIL(BQ_ERR_DTYPE, "float_matmul takes float tensors");
+  auto is_float = [](const bq_tensor* t) { return t->dtype == BQ_F32 || t->dtype == BQ_BF16; };
+  if (!is_float(lhs) || !is_float(rhs)) BQ_FAIL(BQ_ERR_DTYPE, "float_matmul takes float tensors");
   if (lhs->dev != rhs->dev) BQ_FAIL(BQ_ERR_DTYPE, "float_matmul operands live on different devices");
   MatmulDims d;
   BQ_TRY(matmul_dims(lhs, rhs, &d));
@@ -1205,6 +1229,8 @@ static bq_status q_matmul_impl(const bq_tensor* lhs, const bq_tensor* rhs, int32
   BQ_NOTNULL(out);
   const bool lq = lhs->dtype == BQ_QFLOAT, rq = rhs->dtype == BQ_QFLOAT;
   if (!lq && !rq) BQ_FAIL(BQ_ERR_DTYPE, "q_matmul needs at least one quantized operand");
+  if ((!lq && lhs->dtype != BQ_F32 && lhs->dtype != BQ_BF16) || (!rq && rhs->dtype != BQ_F32 && rhs->dtype != BQ_BF16))
+    BQ_FAIL(BQ_ERR_DTYPE, "q_matmul: the operand that is not quantized must be f32 or bf16");
   // dtype any dequantization targets: the float operand's, else f32 (qtensor.rs:507-512)
   const int32_t target = !lq ? lhs->dtype : (!rq ? rhs->dtype : BQ_F32);
   const int32_t out_dtype = out_dtype_req >= 0 ? out_dtype_req : target;
@@ -1614,6 +1640,277 @@ static bq_status q_gather_impl(const bq_tensor* t, const int32_t* axes, const ui
   }
   *out = q;
   return BQ_OK;
+}
+
+// ================================================================================ integer-domain ops
+// q_slice / q_select / q_gather / q_expand / q_argmax / q_argmin on the stored integers, as the reference's CPU
+// backend runs them (crates/burn-ndarray/src/ops/qtensor.rs:349-430): no dequantize, no new scales.
+// One routine builds every result: the values through an index map over the source, the block
+// scales through the same map in block units.
+struct IndexPlan {
+  int rank = 0;                        // of the output
+  size_t out_shape[BQ_MAX_RANK] = {0};
+  int64_t stride[BQ_MAX_RANK] = {0};   // source elements per step of output dim a
+  int64_t base = 0;
+  // block schemes: the same map over the params tensor
+  size_t p_shape[BQ_MAX_RANK] = {0};
+  int64_t p_stride[BQ_MAX_RANK] = {0};
+  int64_t p_base = 0;
+  int index_dim = -1, index_mode = 0;
+  const bq_tensor* indices = nullptr;
+  size_t index_limit = 0;
+};
+
+static bq_status index_map_impl(const bq_tensor* t, const IndexPlan& p, bq_tensor** out) {
+  bq_scheme scheme = t->scheme;
+  // (a Q8S result whose last dim no longer fills whole words is stored natively, as q_permute does)
+  if (scheme.store == BQ_STORE_PACKED_U32 && value_bits(scheme.value) == 8 && p.out_shape[p.rank - 1] % 4 != 0)
+    scheme.store = BQ_STORE_NATIVE;
+  bq_tensor* q = nullptr;
+  BQ_TRY(new_quantized(t->dev, scheme, p.out_shape, p.rank, &q));  // also: "Can't store in u32", dims against the block
+  hipStream_t st = t->dev->stream;
+  const void* idx = p.indices ? p.indices->data : nullptr;
+  const int idx_dtype = p.indices ? p.indices->dtype : BQ_I32;
+  bq_status rc = launch_q_index_map(t->data, q->data, p.out_shape, p.rank, p.stride, p.base, p.index_dim, p.index_mode, idx, idx_dtype,
+                                    p.index_limit, stored_value(t->scheme.value, t->scheme.store), t->scheme.store == BQ_STORE_NATIVE,
+                                    scheme.store == BQ_STORE_NATIVE, st);
+  if (rc == BQ_OK && scheme.level == BQ_LEVEL_BLOCK) {
+    rc = launch_f32_index_map(t->scales(), q->scales(), p.p_shape, p.rank, p.p_stride, p.p_base, p.index_dim, p.index_mode, idx, idx_dtype,
+                              p.index_limit, st);
+    if (rc == BQ_OK && scheme.tensor_scale)
+      rc = launch_f32_index_map(t->wire_scales(), q->wire_scales(), p.p_shape, p.rank, p.p_stride, p.p_base, p.index_dim, p.index_mode, idx,
+                                idx_dtype, p.index_limit, st);
+  } else if (rc == BQ_OK) {
+    hipError_t e = hipMemcpyAsync(q->scales(), t->scales(), 4, hipMemcpyDeviceToDevice, st);
+    if (e != hipSuccess) {
+      set_error("copying the scale failed: %s", hipGetErrorString(e));
+      rc = BQ_ERR_HIP;
+    }
+  }
+  if (rc == BQ_OK && scheme.tensor_scale) {
+    hipError_t e = hipMemcpyAsync(q->wire_global(), t->wire_global(), 4, hipMemcpyDeviceToDevice, st);
+    if (e != hipSuccess) {
+      set_error("copying the per-tensor scale failed: %s", hipGetErrorString(e));
+      rc = BQ_ERR_HIP;
+    }
+  }
+  if (rc != BQ_OK) {
+    bq_tensor_release(q);
+    return rc;
+  }
+  *out = q;
+  return BQ_OK;
+}
+
+static void source_strides(const bq_tensor* t, const size_t* blk, int64_t* stride, int64_t* p_stride) {
+  int64_t s = 1, ps = 1;
+  for (int a = t->rank - 1; a >= 0; --a) {
+    stride[a] = s;
+    p_stride[a] = ps;
+    s *= static_cast<int64_t>(t->shape[a]);
+    ps *= static_cast<int64_t>(t->shape[a] / blk[a]);
+  }
+}
+
+static bq_status check_quantized_for_index_op(const bq_tensor* t, const char* op) {
+  if (t->dtype != BQ_QFLOAT) BQ_FAIL(BQ_ERR_DTYPE, "%s takes a quantized tensor", op);
+  for (int a = 0; a < t->rank; ++a)
+    if (t->shape[a] > 0xFFFFFFFFull) BQ_FAIL(BQ_ERR_SIZE, "%s: dim %d of %zu exceeds 32 bits", op, a, t->shape[a]);
+  return BQ_OK;
+}
+
+// Slice::to_range / output_size (crates/burn-std/src/tensor/slice.rs:493-545): negative indices count
+// from the end, everything is clamped into the dim, a negative step walks the range backwards.
+extern "C" bq_status bq_q_slice(const bq_tensor* t, const int64_t* starts, const int64_t* ends, const int64_t* steps, int32_t n_slices,
+                                bq_tensor** out) {
+  BQ_NOTNULL(t);
+  BQ_NOTNULL(out);
+  BQ_TRY(check_quantized_for_index_op(t, "q_slice"));
+  if (n_slices < 0 || n_slices > t->rank) BQ_FAIL(BQ_ERR_SHAPE, "%d slices for a tensor of rank %d", n_slices, t->rank);
+  if (n_slices > 0) {
+    BQ_NOTNULL(starts);
+    BQ_NOTNULL(ends);
+    BQ_NOTNULL(steps);
+  }
+  size_t blk[BQ_MAX_RANK];
+  block_dims(t->scheme, t->rank, blk);
+  int64_t stride[BQ_MAX_RANK], p_stride[BQ_MAX_RANK];
+  source_strides(t, blk, stride, p_stride);
+  auto signed_index = [](int64_t i, int64_t size) { return i < 0 ? std::max<int64_t>(size + i, 0) : std::min<int64_t>(i, size); };
+  IndexPlan p;
+  p.rank = t->rank;
+  for (int a = 0; a < t->rank; ++a) {
+    const int64_t size = static_cast<int64_t>(t->shape[a]);
+    int64_t start = 0, end = size, step = 1;
+    if (a < n_slices) {
+      step = steps[a];
+      if (step == 0) BQ_FAIL(BQ_ERR_SHAPE, "Step cannot be zero");
+      start = signed_index(starts[a], size);
+      end = ends[a] == INT64_MAX ? size : signed_index(ends[a], size);   // INT64_MAX: to the end of the dim
+    }
+    const int64_t len = end > start ? end - start : 0;
+    const int64_t mag = step < 0 ? -step : step;
+    const int64_t n_out = (len + mag - 1) / mag;
+    const int64_t first = step > 0 ? start : end - 1;
+    p.out_shape[a] = static_cast<size_t>(n_out);
+    p.stride[a] = step * stride[a];
+    p.base += (n_out > 0 ? first : 0) * stride[a];
+    const int64_t b = static_cast<int64_t>(blk[a]);
+    if (b > 1) {
+      // whole blocks only: the scales of the result are the scales of the blocks it keeps
+      if (step != 1 || start % b != 0 || len % b != 0)
+        BQ_FAIL(BQ_ERR_UNSUPPORTED_OP, "q_slice: dim %d is cut inside its blocks of %lld (range %lld..%lld, step %lld)", a,
+                static_cast<long long>(b), static_cast<long long>(start), static_cast<long long>(end), static_cast<long long>(step));
+      p.p_shape[a] = static_cast<size_t>(len / b);
+      p.p_stride[a] = p_stride[a];
+      p.p_base += (start / b) * p_stride[a];
+    } else {
+      p.p_shape[a] = static_cast<size_t>(n_out);
+      p.p_stride[a] = step * p_stride[a];
+      p.p_base += (n_out > 0 ? first : 0) * p_stride[a];
+    }
+  }
+  return index_map_impl(t, p, out);
+}
+
+static bq_status check_indices(const bq_tensor* t, const bq_tensor* indices, const char* op) {
+  BQ_NOTNULL(indices);
+  if (indices->dtype != BQ_I32 && indices->dtype != BQ_I64) BQ_FAIL(BQ_ERR_DTYPE, "%s takes i32 or i64 indices", op);
+  if (indices->dev != t->dev) BQ_FAIL(BQ_ERR_DTYPE, "%s: the indices live on another device", op);
+  return BQ_OK;
+}
+
+extern "C" bq_status bq_q_select(const bq_tensor* t, int32_t dim, const bq_tensor* indices, bq_tensor** out) {
+  BQ_NOTNULL(t);
+  BQ_NOTNULL(out);
+  BQ_TRY(check_quantized_for_index_op(t, "q_select"));
+  BQ_TRY(check_indices(t, indices, "q_select"));
+  if (dim < 0 || dim >= t->rank) BQ_FAIL(BQ_ERR_SHAPE, "q_select: dim %d of a tensor of rank %d", dim, t->rank);
+  if (indices->rank != 1) BQ_FAIL(BQ_ERR_SHAPE, "q_select takes a 1-D index tensor");
+  size_t blk[BQ_MAX_RANK];
+  block_dims(t->scheme, t->rank, blk);
+  if (blk[dim] > 1) BQ_FAIL(BQ_ERR_UNSUPPORTED_OP, "q_select along dim %d would pick single values out of blocks of %zu", dim, blk[dim]);
+  if (t->shape[dim] == 0 && indices->shape[0] > 0) BQ_FAIL(BQ_ERR_SHAPE, "q_select from an empty dim");
+  IndexPlan p;
+  p.rank = t->rank;
+  source_strides(t, blk, p.stride, p.p_stride);
+  for (int a = 0; a < t->rank; ++a) {
+    p.out_shape[a] = a == dim ? indices->shape[0] : t->shape[a];
+    p.p_shape[a] = p.out_shape[a] / blk[a];
+  }
+  p.index_dim = dim;
+  p.index_mode = 1;
+  p.indices = indices;
+  p.index_limit = t->shape[dim];
+  return index_map_impl(t, p, out);
+}
+
+extern "C" bq_status bq_q_gather(int32_t dim, const bq_tensor* t, const bq_tensor* indices, bq_tensor** out) {
+  BQ_NOTNULL(t);
+  BQ_NOTNULL(out);
+  BQ_TRY(check_quantized_for_index_op(t, "q_gather"));
+  BQ_TRY(check_indices(t, indices, "q_gather"));
+  if (dim < 0 || dim >= t->rank) BQ_FAIL(BQ_ERR_SHAPE, "q_gather: dim %d of a tensor of rank %d", dim, t->rank);
+  if (indices->rank != t->rank) BQ_FAIL(BQ_ERR_SHAPE, "q_gather: indices of rank %d for a tensor of rank %d", indices->rank, t->rank);
+  // (the reference folds both operands to [batch, size]: every other dim must agree, base.rs:106-138)
+  for (int a = 0; a < t->rank; ++a)
+    if (a != dim && indices->shape[a] != t->shape[a])
+      BQ_FAIL(BQ_ERR_SHAPE, "q_gather: indices dim %d is %zu, the tensor's is %zu", a, indices->shape[a], t->shape[a]);
+  if (t->scheme.level == BQ_LEVEL_BLOCK) {
+    size_t blk[BQ_MAX_RANK];
+    block_dims(t->scheme, t->rank, blk);
+    for (int a = 0; a < t->rank; ++a)
+      if (blk[a] > 1) BQ_FAIL(BQ_ERR_UNSUPPORTED_OP, "q_gather picks single values: block scales cannot follow them");
+  }
+  if (t->shape[dim] == 0 && indices->numel() > 0) BQ_FAIL(BQ_ERR_SHAPE, "q_gather from an empty dim");
+  size_t blk[BQ_MAX_RANK];
+  block_dims(t->scheme, t->rank, blk);
+  IndexPlan p;
+  p.rank = t->rank;
+  source_strides(t, blk, p.stride, p.p_stride);
+  for (int a = 0; a < t->rank; ++a) p.out_shape[a] = p.p_shape[a] = indices->shape[a];
+  p.index_dim = dim;
+  p.index_mode = 2;
+  p.indices = indices;
+  p.index_limit = t->shape[dim];
+  return index_map_impl(t, p, out);
+}
+
+// Broadcast: trailing dims aligned, a source dim of 1 repeats, new leading dims repeat the whole tensor.
+extern "C" bq_status bq_q_expand(const bq_tensor* t, const size_t* shape, int32_t rank, bq_tensor** out) {
+  BQ_NOTNULL(t);
+  BQ_NOTNULL(shape);
+  BQ_NOTNULL(out);
+  BQ_TRY(check_quantized_for_index_op(t, "q_expand"));
+  if (rank < t->rank || rank > BQ_MAX_RANK) BQ_FAIL(BQ_ERR_SHAPE, "q_expand: rank %d from a tensor of rank %d", rank, t->rank);
+  size_t blk[BQ_MAX_RANK];
+  block_dims(t->scheme, t->rank, blk);
+  int64_t stride[BQ_MAX_RANK], p_stride[BQ_MAX_RANK];
+  source_strides(t, blk, stride, p_stride);
+  IndexPlan p;
+  p.rank = rank;
+  const int lead = rank - t->rank;
+  for (int a = 0; a < rank; ++a) {
+    if (shape[a] > 0xFFFFFFFFull) BQ_FAIL(BQ_ERR_SIZE, "q_expand: dim %d of %zu exceeds 32 bits", a, shape[a]);
+    p.out_shape[a] = shape[a];
+    const int s = a - lead;
+    if (s < 0) {
+      p.stride[a] = p.p_stride[a] = 0;
+      p.p_shape[a] = shape[a];
+    } else if (t->shape[s] == shape[a]) {
+      p.stride[a] = stride[s];
+      p.p_stride[a] = p_stride[s];
+      p.p_shape[a] = shape[a] / blk[s];
+    } else if (t->shape[s] == 1) {   // (a dim of 1 holds blocks of 1)
+      p.stride[a] = p.p_stride[a] = 0;
+      p.p_shape[a] = shape[a];
+    } else {
+      BQ_FAIL(BQ_ERR_SHAPE, "q_expand: dim %d of %zu cannot become %zu", s, t->shape[s], shape[a]);
+    }
+  }
+  return index_map_impl(t, p, out);
+}
+
+static bq_status q_arg_impl(const bq_tensor* t, int32_t dim, int32_t out_dtype, bool want_max, bq_tensor** out) {
+  BQ_NOTNULL(t);
+  BQ_NOTNULL(out);
+  const char* op = want_max ? "q_argmax" : "q_argmin";
+  BQ_TRY(check_quantized_for_index_op(t, op));
+  if (dim < 0 || dim >= t->rank) BQ_FAIL(BQ_ERR_SHAPE, "%s: dim %d of a tensor of rank %d", op, dim, t->rank);
+  if (out_dtype != BQ_I32 && out_dtype != BQ_I64) BQ_FAIL(BQ_ERR_DTYPE, "%s returns i32 or i64 indices", op);
+  // one scale for everything compared: the order of the integers is the order of the values
+  if (t->scheme.level == BQ_LEVEL_BLOCK) {
+    size_t blk[BQ_MAX_RANK];
+    block_dims(t->scheme, t->rank, blk);
+    bool whole = true;
+    for (int a = 0; a < t->rank; ++a) whole = whole && (a == dim ? blk[a] == t->shape[a] : blk[a] == 1);
+    if (!whole) BQ_FAIL(BQ_ERR_UNSUPPORTED_OP, "%s along dim %d compares values of different blocks: dequantize first", op, dim);
+  }
+  if (t->shape[dim] == 0) BQ_FAIL(BQ_ERR_SHAPE, "Cannot compute arg over an empty axis");
+  size_t oshape[BQ_MAX_RANK], outer = 1, inner = 1;
+  for (int a = 0; a < t->rank; ++a) {
+    oshape[a] = a == dim ? 1 : t->shape[a];
+    if (a < dim) outer *= t->shape[a];
+    if (a > dim) inner *= t->shape[a];
+  }
+  bq_tensor* o = nullptr;
+  BQ_TRY(new_float(t->dev, out_dtype, oshape, t->rank, &o));
+  const bq_status rc = launch_q_arg(t->data, stored_value(t->scheme.value, t->scheme.store), t->scheme.store == BQ_STORE_NATIVE, outer,
+                                    t->shape[dim], inner, want_max, out_dtype, o->data, t->dev->stream);
+  if (rc != BQ_OK) {
+    bq_tensor_release(o);
+    return rc;
+  }
+  *out = o;
+  return BQ_OK;
+}
+
+extern "C" bq_status bq_q_argmax(const bq_tensor* t, int32_t dim, int32_t out_dtype, bq_tensor** out) {
+  return q_arg_impl(t, dim, out_dtype, true, out);
+}
+
+extern "C" bq_status bq_q_argmin(const bq_tensor* t, int32_t dim, int32_t out_dtype, bq_tensor** out) {
+  return q_arg_impl(t, dim, out_dtype, false, out);
 }
 
 extern "C" bq_status bq_q_permute(const bq_tensor* t, const int32_t* axes, int32_t rank, bq_tensor** out) {

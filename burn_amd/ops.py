@@ -376,11 +376,80 @@ class QTensorOps:
         return _wrap(h, t.device)
 
     @staticmethod
+    def q_slice(t: Tensor, slices) -> Tensor:
+        """slices: one per leading dim, each a Python slice or an int (a single index keeps the dim, as
+        burn's s![] does); burn's Slice semantics (negative indices, clamping, negative steps)."""
+        n = len(slices)
+        starts, ends, steps = (C.c_int64 * max(n, 1))(), (C.c_int64 * max(n, 1))(), (C.c_int64 * max(n, 1))()
+        for i, s in enumerate(slices):
+            if isinstance(s, int):                     # Slice::index: idx .. idx + 1 (None for -1)
+                s = slice(s, None if s == -1 else s + 1, 1)
+            step = 1 if s.step is None else s.step
+            starts[i] = 0 if s.start is None else s.start
+            ends[i] = (2 ** 63 - 1) if s.stop is None else s.stop
+            steps[i] = step
+        h = C.c_void_p()
+        check(lib().bq_q_slice(t.handle, starts, ends, steps, n, C.byref(h)))
+        return _wrap(h, t.device)
+
+    @staticmethod
+    def q_select(t: Tensor, dim: int, indices: Tensor) -> Tensor:
+        h = C.c_void_p()
+        check(lib().bq_q_select(t.handle, dim, indices.handle, C.byref(h)))
+        return _wrap(h, t.device)
+
+    @staticmethod
+    def q_gather(dim: int, t: Tensor, indices: Tensor) -> Tensor:
+        h = C.c_void_p()
+        check(lib().bq_q_gather(dim, t.handle, indices.handle, C.byref(h)))
+        return _wrap(h, t.device)
+
+    @staticmethod
+    def q_expand(t: Tensor, shape) -> Tensor:
+        sh, rank = _shape_arg(shape)
+        h = C.c_void_p()
+        check(lib().bq_q_expand(t.handle, sh, rank, C.byref(h)))
+        return _wrap(h, t.device)
+
+    @staticmethod
+    def q_argmax(t: Tensor, dim: int, out_dtype: int = _lib.I64) -> Tensor:
+        h = C.c_void_p()
+        check(lib().bq_q_argmax(t.handle, dim, out_dtype, C.byref(h)))
+        return _wrap(h, t.device)
+
+    @staticmethod
+    def q_argmin(t: Tensor, dim: int, out_dtype: int = _lib.I64) -> Tensor:
+        h = C.c_void_p()
+        check(lib().bq_q_argmin(t.handle, dim, out_dtype, C.byref(h)))
+        return _wrap(h, t.device)
+
+    @staticmethod
     def q_flip(t: Tensor, axes: Sequence[int]) -> Tensor:
         arr = (C.c_int32 * max(len(axes), 1))(*axes)
         h = C.c_void_p()
         check(lib().bq_q_flip(t.handle, arr, len(axes), C.byref(h)))
         return _wrap(h, t.device)
+
+
+class IntOps:
+    """The slice of IntTensorOps the quantized index ops need (int_from_data / int_into_data)."""
+
+    @staticmethod
+    def int_from_data(data: np.ndarray, device: Device) -> Tensor:
+        data = np.ascontiguousarray(data)
+        if data.dtype not in (np.int32, np.int64):
+            raise TypeError("index tensors are int32 or int64")
+        shape, rank = _shape_arg(data.shape)
+        h = C.c_void_p()
+        check(lib().bq_int_from_data(device.handle, data.ctypes.data, _lib.I32 if data.dtype == np.int32 else _lib.I64,
+                                     shape, rank, C.byref(h)))
+        return _wrap(h, device)
+
+    @staticmethod
+    def int_into_data(t: Tensor) -> np.ndarray:
+        out = np.empty(t.shape, np.int32 if t.dtype == _lib.I32 else np.int64)
+        check(lib().bq_int_into_data(t.handle, out.ctypes.data, out.nbytes))
+        return out
 
 
 class ModuleOps:

@@ -48,8 +48,9 @@ enum {
   BQ_ERR_NONFINITE = 8           /* validate mode: x / scale is NaN (reference: Q::from(NaN).unwrap() panics) */
 };
 
-/* DType of a handle. BQ_QFLOAT carries a bq_scheme, like DType::QFloat(scheme). */
-enum { BQ_F32 = 0, BQ_BF16 = 1, BQ_QFLOAT = 2 };
+/* DType of a handle. BQ_QFLOAT carries a bq_scheme, like DType::QFloat(scheme). BQ_I32 / BQ_I64 are the
+ * index tensors that q_select / q_gather take and q_argmax / q_argmin return. */
+enum { BQ_F32 = 0, BQ_BF16 = 1, BQ_QFLOAT = 2, BQ_I32 = 3, BQ_I64 = 4 };
 
 /* QuantValue, QuantStore, quantization level (cubecl_common::quant::scheme, re-exported at
  * crates/burn-std/src/tensor/quantization.rs:4-6). The signed-integer values are implemented:
@@ -288,6 +289,41 @@ bq_status bq_q_reshape(const bq_tensor* t, const size_t* shape, int32_t rank, bq
 bq_status bq_q_swap_dims(const bq_tensor* t, int32_t dim1, int32_t dim2, bq_tensor** out);
 bq_status bq_q_permute(const bq_tensor* t, const int32_t* axes, int32_t rank, bq_tensor** out);
 bq_status bq_q_flip(const bq_tensor* t, const int32_t* axes, int32_t n_axes, bq_tensor** out);
+
+/* ------------------------------------------------------------------ integer-domain ops
+ * The QTensorOps methods the reference's CPU backend runs on the stored integers without
+ * dequantizing (crates/burn-ndarray/src/ops/qtensor.rs:349-430; the trait's defaults,
+ * crates/burn-backend/src/backend/ops/qtensor.rs:210-322 and :948-1041, dequantize, run the float op
+ * and quantize again, which changes the scale). The result keeps the source's scheme and scales:
+ * dequantize(op(q)) equals op(dequantize(q)) bit for bit. Block scales follow their blocks where the
+ * op moves whole blocks; where it would cut into blocks the call returns BQ_ERR_UNSUPPORTED_OP and the
+ * binding falls back to the trait's default. A Q8S result whose last dim no longer fills packed words
+ * is stored natively (same bytes), as q_permute does; sub-byte results must fill their words
+ * (BQ_ERR_SHAPE). */
+/* IntTensorOps::int_from_data / int_into_data for index tensors (dtype BQ_I32 or BQ_I64, dense row-major). */
+bq_status bq_int_from_data(bq_device* dev, const void* host, int32_t dtype, const size_t* shape, int32_t rank,
+                           bq_tensor** out);
+bq_status bq_int_into_data(const bq_tensor* t, void* host, size_t capacity_bytes);
+/* QTensorOps::q_slice (qtensor.rs:296): slice a of n_slices is Slice { start: starts[a], end: ends[a] (INT64_MAX for
+ * None), step: steps[a] } with burn's rules (crates/burn-std/src/tensor/slice.rs:493-545): negative indices count from
+ * the end, ranges are clamped into the dim, the output holds ceil(len / |step|) values, a negative step walks the range
+ * backwards from its last value. Dims past n_slices are kept whole. A dim with blocks wider than 1 takes step 1 and
+ * ranges of whole blocks. */
+bq_status bq_q_slice(const bq_tensor* t, const int64_t* starts, const int64_t* ends, const int64_t* steps, int32_t n_slices,
+                     bq_tensor** out);
+/* QTensorOps::q_select (qtensor.rs:274): out[.., i, ..] = t[.., indices[i], ..] along `dim`; indices 1-D. An index outside
+ * the dim, which the reference panics on, is clamped into it. Blocks must be 1 wide along `dim`. */
+bq_status bq_q_select(const bq_tensor* t, int32_t dim, const bq_tensor* indices, bq_tensor** out);
+/* QTensorOps::q_gather (qtensor.rs:312): out[c] = t[c with c[dim] replaced by indices[c]]; indices has t's rank and t's
+ * extents on every other dim (crates/burn-ndarray/src/ops/base.rs:106-138). Per-tensor schemes (or blocks of 1). */
+bq_status bq_q_gather(int32_t dim, const bq_tensor* t, const bq_tensor* indices, bq_tensor** out);
+/* QTensorOps::q_expand (qtensor.rs:210): broadcast to `shape` (trailing dims aligned; a dim of 1 repeats). */
+bq_status bq_q_expand(const bq_tensor* t, const size_t* shape, int32_t rank, bq_tensor** out);
+/* QTensorOps::q_argmax / q_argmin (qtensor.rs:948, :1037): index along `dim` of the largest / smallest value, the first one
+ * on ties (crates/burn-ndarray/src/ops/base.rs:1727-1750), `dim` kept with extent 1; out_dtype BQ_I32 or BQ_I64. Compared
+ * on the integers: per-tensor schemes, or blocks that span exactly the reduced dim. */
+bq_status bq_q_argmax(const bq_tensor* t, int32_t dim, int32_t out_dtype, bq_tensor** out);
+bq_status bq_q_argmin(const bq_tensor* t, int32_t dim, int32_t out_dtype, bq_tensor** out);
 
 /* ------------------------------------------------------------------ burnpack containers
  * The on-disk format quantized modules are saved in (crates/burn-pack: base.rs:13-60 header and

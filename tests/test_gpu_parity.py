@@ -15,7 +15,7 @@ from conftest import burn_approx_eq
 pytestmark = pytest.mark.gpu
 
 import burn_amd as ba  # noqa: E402
-from burn_amd import FloatOps, ModuleOps, QTensorOps, QuantScheme, QuantStore, QuantValue, TensorData  # noqa: E402
+from burn_amd import FloatOps, IntOps, ModuleOps, QTensorOps, QuantScheme, QuantStore, QuantValue, TensorData  # noqa: E402
 from burn_amd.quantization import ScaleDtype  # noqa: E402
 
 VAL = {QuantValue.Q8S: (co.Q8S, "Q8S"), QuantValue.Q4S: (co.Q4S, "Q4S"), QuantValue.Q2S: (co.Q2S, "Q2S"),
@@ -1611,6 +1611,143 @@ def test_burnpack_quantized_entry_of_another_producer(dev):
         t = reader.load(name, dev, scheme=scheme)
         assert t.scheme == scheme and QTensorOps.q_into_data(t).bytes.tobytes() == blobs[name][0].tobytes()
         assert FloatOps.float_into_data(QTensorOps.dequantize(t)).tobytes() == blobs[name][1].tobytes()
+
+
+# ------------------------------------------------------------------ integer-domain ops
+
+REFERENCE_SLICE_CASES = [        # crates/burn-backend-tests/tests/cubecl/quantization/slice.rs:40-128
+    ((8,), (slice(None),)), ((8,), (slice(2, 6),)), ((4, 8), (slice(1, 3), slice(None))), ((4, 8), (slice(None), slice(0, 4))),
+    ((4, 8), (slice(1, 3), slice(4, 8))), ((2, 3, 8), (slice(0, 1), slice(1, 3), slice(None))), ((4, 8), (1, slice(None))),
+    ((4, 8), (slice(1, 3), slice(None))),                    # s![1..=2, ..]
+    ((4, 8), (slice(-2, None), slice(None))), ((4, 8), (slice(None), slice(-4, None))), ((8, 8), (slice(0, 8, 2), slice(None))),
+    ((4, 8), (slice(None), slice(0, 8, 2))), ((4, 8), (slice(None, None, -1), slice(None))), ((4, 8), (slice(None), slice(None, None, -1))),
+    ((4, 8), (slice(1, 3),)),
+]
+
+
+def burn_slice(a, slices):
+    """numpy evaluation of burn's Slice (crates/burn-std/src/tensor/slice.rs:493-545): the range start..end is
+    normalised first (negative indices from the end, clamped), then walked with the step -- backwards from its last
+    element when the step is negative."""
+    out = a
+    for d, s in enumerate(slices):
+        size = a.shape[d]
+        if isinstance(s, int):
+            s = slice(s, None if s == -1 else s + 1, 1)
+        conv = lambda i: max(size + i, 0) if i < 0 else min(i, size)   # noqa: E731
+        start = 0 if s.start is None else conv(s.start)
+        end = size if s.stop is None else conv(s.stop)
+        step = 1 if s.step is None else s.step
+        idx = np.arange(start, max(end, start))
+        idx = idx[::step] if step > 0 else idx[::-1][::-step]
+        out = np.take(out, idx, axis=d)
+    return out
+
+
+@pytest.mark.parametrize("shape,slices", REFERENCE_SLICE_CASES)
+def test_q_slice_reference_cases(dev, shape, slices):
+    """The reference's q_slice cases (arange / numel, its default scheme: Q8F per tensor, packed): slicing
+    the quantized tensor and dequantizing equals dequantizing and slicing -- bit for bit here, where the
+    reference allows Tolerance::permissive() -- and the integers are the sliced integers."""
+    numel = int(np.prod(shape))
+    x = (np.arange(numel, dtype=np.float32) / np.float32(numel)).reshape(shape)
+    scheme = QuantScheme(value=QuantValue.Q8F)
+    tq = QTensorOps.quantize_dynamic(FloatOps.float_from_data(x, dev), scheme)
+    q_ref, s_ref = co.quantize_dynamic(x, oscheme(scheme))
+    want = burn_slice(co.dequantize(q_ref, oscheme(scheme), s_ref), slices)
+    got_t = QTensorOps.q_slice(tq, slices)
+    assert got_t.shape == want.shape and got_t.scheme == scheme
+    got = FloatOps.float_into_data(QTensorOps.dequantize(got_t))
+    assert got.tobytes() == np.ascontiguousarray(want).tobytes()
+    q, s = unpack_blob(QTensorOps.q_into_data(got_t))
+    assert (q == burn_slice(q_ref, slices)).all() and s.tobytes() == s_ref.tobytes()
+
+
+@pytest.mark.parametrize("value", [QuantValue.Q8S, QuantValue.Q4S, QuantValue.Q2S])
+@pytest.mark.parametrize("store", [QuantStore.PackedU32, QuantStore.Native])
+def test_integer_domain_ops_against_numpy(dev, value, store):
+    """q_slice / q_select / q_gather / q_expand / q_argmax / q_argmin (crates/burn-ndarray/src/ops/qtensor.rs:349-430)
+    on seeded tensors, per tensor and per block: the result's integers are numpy's op on the oracle's
+    integers, its scales the op on the scales (in block units), the scheme unchanged."""
+    rng = np.random.default_rng(11 + 3 * int(value == QuantValue.Q4S) + int(store == QuantStore.Native))
+    x = awkward((6, 8, 64), 77)
+    for block in (None, (32,), (2, 1, 16)):
+        scheme = QuantScheme(value=value, store=store) if block is None else QuantScheme(value=value, store=store).per_block(block)
+        tq = QTensorOps.quantize_dynamic(FloatOps.float_from_data(x, dev), scheme)
+        q_ref, s_ref = co.quantize_dynamic(x, oscheme(scheme))
+        blk = (1, 1, 1) if block is None else tuple([1] * (3 - len(block)) + list(block))
+
+        def check(t, q_want, s_want):
+            q, s = unpack_blob(QTensorOps.q_into_data(t))
+            assert t.shape == q_want.shape and (q == q_want).all()
+            assert s.reshape(-1).tobytes() == np.ascontiguousarray(s_want, np.float32).reshape(-1).tobytes()
+            d = FloatOps.float_into_data(QTensorOps.dequantize(t))
+            return d
+
+        pshape = [6 // blk[0], 8 // blk[1], 64 // blk[2]]
+        s_elem = np.kron(s_ref.reshape(pshape), np.ones(blk, np.float32)) if block is not None else None   # one scale per element
+
+        def scales_of(op):               # the op on the per-element scales, one value kept per block
+            return s_ref if block is None else op(s_elem)[::blk[0], ::blk[1], ::blk[2]]
+
+        # slices that keep whole blocks and whole packed words
+        for slices in ((slice(2, 6), slice(None), slice(32, 64)), (slice(None, None, 1), slice(3, 8), slice(None)),
+                       (slice(0, 2), 5, slice(0, 32)), (slice(-4, None), slice(None, None, -1), slice(None))):
+            d = check(QTensorOps.q_slice(tq, slices), burn_slice(q_ref, slices), scales_of(lambda a: burn_slice(a, slices)))
+            assert d.tobytes() == np.ascontiguousarray(burn_slice(co.dequantize(q_ref, oscheme(scheme), s_ref), slices)).tobytes()
+        # a cut inside a block is declined (the trait's default takes over)
+        if block is not None:
+            with pytest.raises(ba.BurnqError) as e:
+                QTensorOps.q_slice(tq, (slice(None), slice(None), slice(8, 40)))
+            assert e.value.status == ba._lib.ERR_UNSUPPORTED_OP
+        # select along a dim whose blocks are 1 wide
+        idx = rng.integers(0, 8, 5)
+        for np_idx in (idx.astype(np.int32), idx.astype(np.int64)):
+            check(QTensorOps.q_select(tq, 1, IntOps.int_from_data(np_idx, dev)), np.take(q_ref, idx, axis=1),
+                  scales_of(lambda a: np.take(a, idx, axis=1)))
+        # expand: new leading dims
+        check(QTensorOps.q_expand(tq, (3, 6, 8, 64)), np.broadcast_to(q_ref, (3, 6, 8, 64)),
+              s_ref if block is None else np.broadcast_to(s_ref.reshape(pshape), [3] + pshape))
+        if block is None:
+            # gather along every dim, and a dim of 1 broadcast
+            for dim in range(3):
+                shape = list(x.shape)
+                shape[dim] = 16 if dim == 2 else 4     # whole packed words along the last dim
+                gi = rng.integers(0, x.shape[dim], shape)
+                check(QTensorOps.q_gather(dim, tq, IntOps.int_from_data(gi.astype(np.int64), dev)), np.take_along_axis(q_ref, gi, axis=dim), s_ref)
+            one = QTensorOps.q_slice(tq, (slice(None), slice(2, 3), slice(None)))
+            check(QTensorOps.q_expand(one, (6, 5, 64)), np.broadcast_to(q_ref[:, 2:3, :], (6, 5, 64)), s_ref)
+            for dim in range(3):
+                for dtype, npd in ((ba.I32, np.int32), (ba.I64, np.int64)):
+                    am = IntOps.int_into_data(QTensorOps.q_argmax(tq, dim, dtype))
+                    an = IntOps.int_into_data(QTensorOps.q_argmin(tq, dim, dtype))
+                    assert am.dtype == npd and (am == np.expand_dims(q_ref.argmax(axis=dim), dim)).all()
+                    assert (an == np.expand_dims(q_ref.argmin(axis=dim), dim)).all()
+            # the arg over the integers is the arg over the dequantized values
+            deq = co.dequantize(q_ref, oscheme(scheme), s_ref)
+            assert (IntOps.int_into_data(QTensorOps.q_argmax(tq, 2)) == np.expand_dims(deq.argmax(axis=2), 2)).all()
+        else:
+            with pytest.raises(ba.BurnqError) as e:
+                QTensorOps.q_gather(0, tq, IntOps.int_from_data(np.zeros((2, 8, 64), np.int64), dev))
+            assert e.value.status == ba._lib.ERR_UNSUPPORTED_OP
+            with pytest.raises(ba.BurnqError) as e:
+                QTensorOps.q_argmax(tq, 2)
+            assert e.value.status == ba._lib.ERR_UNSUPPORTED_OP
+    # results that do not fill packed words: Q8S goes native with the same bytes, sub-byte values are refused
+    tq = QTensorOps.quantize_dynamic(FloatOps.float_from_data(x, dev), QuantScheme(value=value, store=store))
+    q_ref, s_ref = co.quantize_dynamic(x, oscheme(QuantScheme(value=value, store=store)))
+    if value == QuantValue.Q8S or store == QuantStore.Native:
+        t = QTensorOps.q_slice(tq, (slice(None), slice(None), slice(1, 4)))
+        q, s = unpack_blob(QTensorOps.q_into_data(t))
+        assert t.scheme.store == QuantStore.Native and (q == q_ref[:, :, 1:4]).all()
+    else:
+        with pytest.raises(ba.BurnqError) as e:
+            QTensorOps.q_slice(tq, (slice(None), slice(None), slice(1, 4)))
+        assert e.value.status == ba._lib.ERR_SHAPE
+    # out-of-range indices are clamped, never a fault
+    far = IntOps.int_from_data(np.int64([-5, 0, 7, 100]), dev)
+    q, _ = unpack_blob(QTensorOps.q_into_data(QTensorOps.q_select(tq, 1, far)))
+    assert (q == np.take(q_ref, [0, 0, 7, 7], axis=1)).all()
 
 
 # ------------------------------------------------------------------ Calibration::AbsMean
