@@ -111,8 +111,24 @@ __device__ __forceinline__ float quad_lane(uint32_t v) {
 template <int VPL, bool PER_TENSOR, bool X_BF16, int MT, int SB = 0, bool PK = false, bool DL = false>
 __global__ void __launch_bounds__(kSplitThreads)
 qsplit_kernel(const void* __restrict__ x, const uint32_t* __restrict__ w, const float* __restrict__ scales,
-              size_t M, size_t K, size_t N, size_t k_per_wg, float* __restrict__ part) {
+              size_t M, size_t K, size_t N, size_t k_per_wg, unsigned tiles, unsigned slices, float* __restrict__ part) {
   extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
+  // Workgroup -> (column tile, K slice). Workgroups reach the 8 XCDs round robin (workgroup b runs
+  // on XCD b % 8) and each XCD has its own L2. A 128-byte line of scales serves kBundle adjacent
+  // column tiles of one K slice: those tiles are given to consecutive workgroups of ONE XCD, so the
+  // line comes from HBM once instead of once per XCD that holds one of its tiles (with the plain
+  // (tile, slice) grid, neighbouring tiles sat on neighbouring XCDs and the scales were read twice:
+  // 1.12 to 1.15 times the weights' bytes by the counters).
+  constexpr unsigned kBundle = PER_TENSOR ? 1u : (2u << SB);
+  unsigned tile_id, slice_id;
+  {
+    const unsigned b = blockIdx.x, xcd = b % 8u, local = b / 8u;
+    const unsigned bundles = (tiles + kBundle - 1u) / kBundle;
+    const unsigned unit = xcd + 8u * (local / kBundle);
+    tile_id = (unit % bundles) * kBundle + local % kBundle;
+    slice_id = unit / bundles;
+    if (slice_id >= slices || tile_id >= tiles) return;  // padding of the grid (whole workgroup)
+  }
   // Activation slice as [16 rows][k_per_wg + 4] f32: the pitch is 4 floats past a multiple of 64,
   // so the 16 rows read by a quarter wave (16 bytes each) fall into distinct banks. The same
   // memory carries the cross-wave sum afterwards.
@@ -136,11 +152,11 @@ qsplit_kernel(const void* __restrict__ x, const uint32_t* __restrict__ w, const 
   const int c = lane & 15, kg = lane >> 4;
   const int g = wave % kGroups, h = wave / kGroups;
   const size_t NW = N / VPL, spr = N / (32u << SB), groups_total = N / kGroupCols;
-  const size_t group = static_cast<size_t>(blockIdx.x) * kGroups + g;
+  const size_t group = static_cast<size_t>(tile_id) * kGroups + g;
   const bool live = group < groups_total;  // the last tile may hold fewer than 4 groups: the spare
   const size_t gc = live ? group : groups_total - 1;  // waves redo the last one and store nothing
 
-  const size_t k_begin = static_cast<size_t>(blockIdx.y) * k_per_wg;
+  const size_t k_begin = static_cast<size_t>(slice_id) * k_per_wg;
   const uint32_t k_per_way = static_cast<uint32_t>(k_per_wg) / kKWays;
   const size_t kw0 = k_begin + static_cast<size_t>(h) * k_per_way;  // first row of this wave
   const int steps = kw0 < K ? static_cast<int>((K - kw0 < k_per_way ? K - kw0 : k_per_way) / kStepRows) : 0;
@@ -539,8 +555,8 @@ qsplit_kernel(const void* __restrict__ x, const uint32_t* __restrict__ w, const 
   }
   __syncthreads();
   {
-    float* dst = part + static_cast<size_t>(blockIdx.y) * M * N;
-    const size_t tile_col0 = static_cast<size_t>(blockIdx.x) * kTileCols;
+    float* dst = part + static_cast<size_t>(slice_id) * M * N;
+    const size_t tile_col0 = static_cast<size_t>(tile_id) * kTileCols;
 #pragma unroll
     for (int r = 0; r < 4 * MT; ++r) {
       const uint32_t idx = static_cast<uint32_t>(tid) + static_cast<uint32_t>(r) * kSplitThreads;
@@ -591,13 +607,16 @@ bq_status launch_qsplit(const void* x, int x_dtype, const uint32_t* w, const flo
   const bool per_tensor = block == 0;
   const size_t mt = m > 16 ? 2 : 1;
   const size_t lds = 16 * mt * (kMaxSlice + 4) * sizeof(float) + kSplitWaves * kSlotBytes;
-  dim3 grid(p.tiles, p.slices), tb(kSplitThreads);
+  dim3 tb(kSplitThreads);
 #define BQ_SPLIT3(V, PT, XB, T, S, P)                                                              \
   do {                                                                                            \
     auto kernel = qsplit_kernel<V, PT, XB, T, S, P, (P || PT)>;                                            \
+    /* the kernel's workgroup map: bundles of adjacent tiles, dealt to the XCDs 8 at a time */    \
+    const unsigned bundle = PT ? 1u : (2u << S), units = (p.tiles + bundle - 1u) / bundle * p.slices;  \
+    dim3 grid(8u * bundle * ((units + 7u) / 8u));                                                 \
     /* more than the default 64 KiB: checked against what the device grants, else refused here */ \
     BQ_TRY(configure_dynamic_lds(reinterpret_cast<const void*>(kernel), lds, "qsplit_kernel"));   \
-    hipLaunchKernelGGL(kernel, grid, tb, lds, st, x, w, scales, m, k, n, p.k_per_wg, part);       \
+    hipLaunchKernelGGL(kernel, grid, tb, lds, st, x, w, scales, m, k, n, p.k_per_wg, p.tiles, p.slices, part);       \
   } while (0)
 #define BQ_SPLIT(V, PT, XB, S)                  \
   if (mt == 2) BQ_SPLIT3(V, PT, XB, 2, S, false); else BQ_SPLIT3(V, PT, XB, 1, S, false)
