@@ -1750,6 +1750,61 @@ def test_integer_domain_ops_against_numpy(dev, value, store):
     assert (q == np.take(q_ref, [0, 0, 7, 7], axis=1)).all()
 
 
+def _int8(dev, floats):
+    """The reference tests' QTensor::int8: quantize_dynamic, Q8S per tensor (native store, as the backends
+    that run them; crates/burn-backend-tests/tests/tensor/float/quantization/mod.rs:23-50)."""
+    x = np.asarray(floats, np.float32)
+    return QTensorOps.quantize_dynamic(FloatOps.float_from_data(x, dev), QuantScheme(value=QuantValue.Q8S, store=QuantStore.Native))
+
+
+def _deq(t):
+    return FloatOps.float_into_data(QTensorOps.dequantize(t))
+
+
+def test_q_arg_expand_select_gather_reference_cases(dev):
+    """The reference's own cases for the integer-domain ops
+    (crates/burn-backend-tests/tests/tensor/float/quantization/ops/extended/{arg,expand,select,gather_scatter}.rs),
+    inputs and expected outputs as written there, with the tolerance each of them states."""
+    # arg.rs:6-50
+    a = [[10.0, 11.0, 2.0], [3.0, 4.0, 5.0]]
+    b = [[10.0, 11.0, 2.0], [30.0, 4.0, 5.0]]
+    assert IntOps.int_into_data(QTensorOps.q_argmax(_int8(dev, a), 0)).tolist() == [[0, 0, 1]]
+    assert IntOps.int_into_data(QTensorOps.q_argmin(_int8(dev, b), 0)).tolist() == [[0, 1, 0]]
+    assert IntOps.int_into_data(QTensorOps.q_argmax(_int8(dev, a), 1)).tolist() == [[1], [2]]
+    assert IntOps.int_into_data(QTensorOps.q_argmin(_int8(dev, b), 1)).tolist() == [[2], [1]]
+    # expand.rs:7-100 (Tolerance::absolute(1e-1); the single-value broadcast is exact)
+    for src, shape in (([1.0, 2.0, 3.0], (3, 3)), ([4.0, 7.0, 2.0, 3.0], (2, 4)), ([[1.0, 2.0], [3.0, 4.0]], (3, 2, 2)),
+                       ([[1.0, 2.0, 3.0, 4.0]], (2, 3, 4))):
+        got = _deq(QTensorOps.q_expand(_int8(dev, src), shape))
+        assert got.shape == shape and np.abs(got - np.broadcast_to(np.float32(src), shape)).max() <= 1e-1
+    assert _deq(QTensorOps.q_expand(_int8(dev, [1.0]), (2, 3))).tolist() == [[1.0, 1.0, 1.0], [1.0, 1.0, 1.0]]
+    with pytest.raises(ba.BurnqError) as e:                      # should_fail_expand_incompatible_shapes
+        QTensorOps.q_expand(_int8(dev, [1.0, 2.0, 3.0]), (2, 2))
+    assert e.value.status == ba._lib.ERR_SHAPE
+    # select.rs:8-70 (Tolerance::rel_abs(2e-2, 1e-2))
+    for src, dim, idx, want in (
+            ([0.0, 1.0, 2.0, 3.0], 0, [1, 1, 0, 1, 2], [1.0, 1.0, 0.0, 1.0, 2.0]),
+            ([[0.0, 1.0, 2.0], [3.0, 4.0, 5.0]], 0, [1, 0], [[3.0, 4.0, 5.0], [0.0, 1.0, 2.0]]),
+            ([[0.0, 1.0, 2.0], [3.0, 4.0, 5.0]], 0, [1, 0, 1, 1], [[3.0, 4.0, 5.0], [0.0, 1.0, 2.0], [3.0, 4.0, 5.0], [3.0, 4.0, 5.0]]),
+            ([[0.0, 1.0, 2.0], [3.0, 4.0, 5.0]], 1, [1, 1, 0, 1, 2], [[1.0, 1.0, 0.0, 1.0, 2.0], [4.0, 4.0, 3.0, 4.0, 5.0]])):
+        got = _deq(QTensorOps.q_select(_int8(dev, src), dim, IntOps.int_from_data(np.int64(idx), dev)))
+        want = np.float32(want)
+        assert got.shape == want.shape and (np.abs(got - want) <= 1e-2 + 2e-2 * np.abs(want)).all()
+    # gather_scatter.rs:8-100 (Tolerance::absolute(1e-1))
+    m23 = [[0.0, 1.0, 2.0], [3.0, 4.0, 5.0]]
+    for src, dim, idx, want in (
+            ([0.0, 1.0, 2.0], 0, [1, 1, 0, 1, 2], [1.0, 1.0, 0.0, 1.0, 2.0]),
+            (m23, 0, [[0, 1, 0], [1, 0, 1]], [[0.0, 4.0, 2.0], [3.0, 1.0, 5.0]]),
+            (m23, 1, [[2, 1, 0, 0], [2, 0, 1, 2]], [[2.0, 1.0, 0.0, 0.0], [5.0, 3.0, 4.0, 5.0]]),
+            ([[[0.0, 1.0, 2.0], [3.0, 4.0, 5.0]], [[6.0, 7.0, 8.0], [9.0, 10.0, 11.0]]], 1,
+             [[[1, 0, 0], [0, 1, 0]], [[0, 0, 1], [0, 1, 1]]],
+             [[[3.0, 1.0, 2.0], [0.0, 4.0, 2.0]], [[6.0, 7.0, 11.0], [6.0, 10.0, 11.0]]]),
+            (m23, 1, [[1], [2]], [[1.0], [5.0]])):
+        got = _deq(QTensorOps.q_gather(dim, _int8(dev, src), IntOps.int_from_data(np.int64(idx), dev)))
+        want = np.float32(want)
+        assert got.shape == want.shape and np.abs(got - want).max() <= 1e-1
+
+
 # ------------------------------------------------------------------ Calibration::AbsMean
 
 def test_abs_mean_calibration_reference_cases(dev, kats, approx):
