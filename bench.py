@@ -41,10 +41,12 @@ MEASURED_TRAFFIC_BYTES = {
     "absmax_kernel + quantize_tensor_kernel<4,from_absmax>": 151143800,    # both passes; algorithmic 150994948
     "dequantize_kernel<4,f32> per tensor": 83885773,                       # algorithmic 83886084
     "dequantize_kernel<8,f32>": 271535104,                                 # algorithmic 271581184
-    # the main kernel of each pair (weights + scales 66060288; the reduction adds about 1 / 3.6 / 8.1 MB)
-    "qgemv1_kernel<4,block,1> + qgemv_reduce_kernel": 67180032,
-    "qsplit_kernel<4,block,f32,row-packed> + qgemv_reduce_kernel": 75915674,
-    "qsplit_kernel<4,block,f32> + qgemv_reduce_kernel": 83001139,
+    # weights + scales are 66060288. M = 1 is one launch (the last workgroup of a strip sums the K slices: the
+    # partial sums written and read back are in the figure); M = 4 / 16: the main kernel of the pair (the
+    # reduction launch adds about 2.1 / 8.3 MB)
+    "qgemv1_kernel<4,block,1> (one launch: the last workgroup of a strip sums the K slices)": 68192000,            # 67.21 MB read + 0.98 MB written
+    "qsplit_kernel<4,block,f32,row-packed> + qgemv_reduce_kernel": 68551000,   # 66.72 MB read + 1.83 MB written
+    "qsplit_kernel<4,block,f32> + qgemv_reduce_kernel": 75667000,             # 68.33 MB read + 7.34 MB written
     "qgemm_kernel<8,256,f32>": 333632000,   # 216.3 MB read (activations + weights + scales are 53.5 MB) + 117.4 MB written
 }
 METRIC = "quant/dequant + q-GEMV GB/s (% HBM peak); prefill q-GEMM TFLOP/s (% MFMA)"
@@ -374,7 +376,7 @@ def run_c4(ba, dev, steps, warmup, cpu):
            "parity": "512 sampled columns of every timed product vs float64 x . dequantize(W): max-normalised "
                      "error <= 1e-2 and burn's permissive rule on every element",
            "weight_bytes": weight_bytes}
-    kernels = {1: "qgemv1_kernel<4,block,1> + qgemv_reduce_kernel", 4: "qsplit_kernel<4,block,f32,row-packed> + qgemv_reduce_kernel",
+    kernels = {1: "qgemv1_kernel<4,block,1> (one launch: the last workgroup of a strip sums the K slices)", 4: "qsplit_kernel<4,block,f32,row-packed> + qgemv_reduce_kernel",
                16: "qsplit_kernel<4,block,f32> + qgemv_reduce_kernel"}
     for m in (1, 4, 16):
         xh = normal_f32(100 + m, (m, k))
