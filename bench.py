@@ -706,6 +706,64 @@ def run_next(ba, dev, steps, warmup, cpu):
                                  "the new last dim, scales moved with their blocks",
                      "parity": "values and scales bit-exact vs the transposed oracle tensor, 256 x 8192",
                      "swap_dims": {"ms": t_t, "GB/s": b / t_t / 1e6, "frac_hbm": b / t_t / 1e6 / HBM_PEAK_GBS, "bytes": b}}
+    # ---- integer-domain ops on the same packed tensors ------------------------------------------------
+    from burn_amd import IntOps
+    import burn_amd as _ba
+    idx_h = np.random.default_rng(0x5E1).integers(0, 256, 192)
+    sl = (slice(32, 224), slice(2048, 6144))
+    got = QTensorOps.q_into_data(QTensorOps.q_slice(tq_small, sl))
+    gv, gs = got.split()
+    if no.unpack_u32(gv.view(np.uint32), got.shape, "Q8S").tobytes() != np.ascontiguousarray(q_ref[sl]).tobytes() or \
+            gs.reshape(-1).tobytes() != np.ascontiguousarray(s_ref.reshape(256, 256)[32:224, 64:192]).tobytes():
+        raise ParityError("q_slice of a packed block-quantized tensor differs from the sliced oracle tensor")
+    got = QTensorOps.q_into_data(QTensorOps.q_select(tq_small, 0, IntOps.int_from_data(idx_h.astype(np.int64), dev)))
+    gv, gs = got.split()
+    if no.unpack_u32(gv.view(np.uint32), got.shape, "Q8S").tobytes() != np.ascontiguousarray(q_ref[idx_h]).tobytes() or \
+            gs.reshape(-1).tobytes() != np.ascontiguousarray(s_ref.reshape(256, 256)[idx_h]).tobytes():
+        raise ParityError("q_select of a packed block-quantized tensor differs from the oracle's rows")
+    t_sl = graph_ms(dev, lambda: [QTensorOps.q_slice(q, (slice(1024, 7168), slice(2048, 6144))) for q in qs], 8, steps, warmup)
+    b_sl = 2 * (6144 * 4096 + 4 * 6144 * 4096 // 32)
+    rows_idx = IntOps.int_from_data(np.random.default_rng(0x5E2).integers(0, rows, rows).astype(np.int64), dev)
+    t_se = graph_ms(dev, lambda: [QTensorOps.q_select(q, 0, rows_idx) for q in qs], 8, steps, warmup)
+    b_se = 2 * (nel + 4 * nel // 32) + 8 * rows
+    pt = QuantScheme()                                                   # Q8S per tensor, packed
+    osch_pt = co.Scheme.make(co.Q8S, None, co.STORE_PACKED_U32)
+    q_pt, _ = co.quantize_dynamic(small, osch_pt)
+    am = IntOps.int_into_data(QTensorOps.q_argmax(QTensorOps.quantize_dynamic(FloatOps.float_from_data(small, dev), pt), 1))
+    if am.reshape(-1).tolist() != q_pt.argmax(axis=1).tolist():
+        raise ParityError("q_argmax differs from the first maximum of the oracle's integers")
+    qpt = [QTensorOps.quantize_dynamic(xs[i % 5], pt) for i in range(8)]
+    t_am = graph_ms(dev, lambda: [QTensorOps.q_argmax(q, 1) for q in qpt], 8, steps, warmup)
+    b_am = nel + 8 * rows
+    out["integer_domain"] = {
+        "workload": "q_slice [1024:7168, 2048:6144], q_select of 8192 random rows (dim 0) of a Q8S block-32 PackedU32 [8192,8192] "
+                    "tensor, values and scales moved together; q_argmax along the last dim of the per-tensor one",
+        "parity": "integers and scales bit-exact vs numpy on the oracle's tensor, 256 x 8192",
+        "q_slice": {"ms": t_sl, "GB/s": b_sl / t_sl / 1e6, "frac_hbm": b_sl / t_sl / 1e6 / HBM_PEAK_GBS, "bytes": b_sl},
+        "q_select": {"ms": t_se, "GB/s": b_se / t_se / 1e6, "frac_hbm": b_se / t_se / 1e6 / HBM_PEAK_GBS, "bytes": b_se},
+        "q_argmax": {"ms": t_am, "GB/s": b_am / t_am / 1e6, "frac_hbm": b_am / t_am / 1e6 / HBM_PEAK_GBS, "bytes": b_am}}
+    del qpt, rows_idx
+    dev.trim()
+
+    # ---- Calibration::AbsMean: the ranges of a ternary weight ------------------------------------------
+    tsch_am = QuantScheme(value=QuantValue.Q2S)
+    osch_t = co.Scheme.make(co.Q2S, None, co.STORE_PACKED_U32)
+    g_ref = co.compute_range_abs_mean(small, osch_t)[1].reshape(-1)[0]
+    tq_am = QTensorOps.quantize_abs_mean(FloatOps.float_from_data(small, dev), tsch_am)
+    av, a_s = QTensorOps.q_into_data(tq_am).split()
+    g_gpu = a_s.reshape(-1)
+    # the mean is a sum the reference leaves to its backend (no order to match): Tolerance::default() between the
+    # two, then everything computed from the device's own scale bit for bit
+    if abs(float(g_gpu[0]) - float(g_ref)) > 1e-5 * abs(float(g_ref)):    # scale = 2 gamma / 2
+        raise ParityError("AbsMean: gamma differs from the oracle's beyond a rounding of the sum")
+    if no.unpack_u32(av.view(np.uint32), small.shape, "Q2S").tobytes() != co.quantize(small, osch_t, g_gpu.copy()).tobytes():
+        raise ParityError("AbsMean: the integers differ from the oracle's quantize with the same scale")
+    t_am2 = graph_ms(dev, lambda: [QTensorOps.quantize_abs_mean(xs[i % 5], tsch_am) for i in range(10)], 10, steps, warmup)
+    b_am2 = 4 * nel + 4 * nel + nel // 4 + 4
+    out["abs_mean"] = {"workload": "C2's tensor -> Q2S per tensor PackedU32 with Calibration::AbsMean: mean |x| (one pass), then quantize",
+                       "parity": "gamma within 1e-5 of the oracle's f64 mean; integers bit-exact vs the oracle's quantize with the device's scale, 256 x 8192",
+                       "quantize_abs_mean": {"ms": t_am2, "GB/s": b_am2 / t_am2 / 1e6, "frac_hbm": b_am2 / t_am2 / 1e6 / HBM_PEAK_GBS,
+                                             "bytes": b_am2, "note": "two passes over x: 4N + 4N + N/4 bytes"}}
     del qs, xs
     dev.trim()
 

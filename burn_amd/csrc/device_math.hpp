@@ -129,6 +129,11 @@ __device__ __forceinline__ uint32_t pack_fields(const int (&q)[VPL]) {
     const uint32_t lo = __builtin_amdgcn_perm(static_cast<uint32_t>(q[1]), static_cast<uint32_t>(q[0]), 0x0c0c0400u);
     const uint32_t hi = __builtin_amdgcn_perm(static_cast<uint32_t>(q[3]), static_cast<uint32_t>(q[2]), 0x04000c0cu);
     return lo | hi;
+  } else if (VPL == 16) {
+    uint32_t w = 0;
+#pragma unroll
+    for (int i = 0; i < 16; ++i) w |= (static_cast<uint32_t>(q[i]) & 0x3u) << (2 * i);
+    return w;
   } else {
     uint32_t b[4];
 #pragma unroll

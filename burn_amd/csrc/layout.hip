@@ -282,6 +282,100 @@ f32_index_map_kernel(const float* __restrict__ src, float* __restrict__ dst, siz
   if (e < n) dst[e] = src[mapped_index(d, e, indices)];
 }
 
+// Fast path of the index maps: the innermost output dim walks the source with stride 1 and carries
+// no index, so an output row is one contiguous run of source bytes (a slice, select or expand that
+// leaves the last dim alone, or cuts it at word boundaries). A lane copies 16 (or 4) bytes; the
+// row's coordinates come from divisions by constants the host prepared (q = (n * m) >> s, exact for
+// n < 2^31), a few instructions per dim instead of a 64-bit division each.
+struct FastDiv {
+  uint32_t m, s, d;
+};
+__device__ __forceinline__ uint32_t fast_div(uint32_t n, const FastDiv& f) {
+  return static_cast<uint32_t>((static_cast<uint64_t>(n) * f.m) >> f.s);
+}
+struct RowMap {
+  int rank;                        // outer dims (output rank - 1)
+  FastDiv div[BQ_MAX_RANK];        // by the extent of outer dim a
+  int64_t stride[BQ_MAX_RANK];     // source bytes per step of outer dim a
+  int64_t base;                    // source byte offset of the first row
+  FastDiv per_row;                 // by the vectors per row
+  int index_dim;                   // outer dim whose coordinate goes through `indices`, or -1
+  int index_i64;
+  int64_t index_limit;
+};
+
+template <typename V>
+__global__ void __launch_bounds__(256)
+row_copy_kernel(const unsigned char* __restrict__ src, unsigned char* __restrict__ dst, uint32_t total, RowMap d,
+                const void* __restrict__ indices) {
+  const uint32_t u = blockIdx.x * 256u + threadIdx.x;
+  if (u >= total) return;
+  const uint32_t row = fast_div(u, d.per_row), v = u - row * d.per_row.d;
+  int64_t off = d.base + static_cast<int64_t>(v) * static_cast<int64_t>(sizeof(V));
+  uint32_t rem = row;
+  for (int a = d.rank - 1; a >= 0; --a) {
+    const uint32_t q = fast_div(rem, d.div[a]);
+    int64_t i = static_cast<int64_t>(rem - q * d.div[a].d);
+    rem = q;
+    if (a == d.index_dim) {
+      i = d.index_i64 ? static_cast<const int64_t*>(indices)[i] : static_cast<int64_t>(static_cast<const int32_t*>(indices)[i]);
+      i = i < 0 ? 0 : (i >= d.index_limit ? d.index_limit - 1 : i);
+    }
+    off += i * d.stride[a];
+  }
+  const V val = __builtin_nontemporal_load(reinterpret_cast<const V*>(src + off));
+  __builtin_nontemporal_store(val, reinterpret_cast<V*>(dst) + u);
+}
+
+// Arg max / min along the last dim of 8-bit values: a wave per row. A lane walks the row 16 bytes at
+// a time keeping its first best; the wave then takes the best of 64 (value, then lowest index) keys.
+__global__ void __launch_bounds__(256)
+q8_arg_last_kernel(const int8_t* __restrict__ src, size_t rows, size_t len, bool want_max, bool out_i64, void* __restrict__ out) {
+  const size_t row = static_cast<size_t>(blockIdx.x) * 4 + threadIdx.x / kWave;
+  if (row >= rows) return;
+  const int lane = threadIdx.x & (kWave - 1);
+  const int8_t* p = src + row * len;
+  int best = want_max ? -129 : 128;
+  uint32_t best_at = 0xFFFFFFFFu;
+  auto take = [&](int v, uint32_t at) {
+    if (want_max ? v > best : v < best) {
+      best = v;
+      best_at = at;
+    }
+  };
+  const bool vec = (reinterpret_cast<uintptr_t>(p) & 15u) == 0;
+  const size_t whole = vec ? len / 16 * 16 : 0;
+  auto take16 = [&](const vuint4& w, size_t i) {
+    const uint32_t ws[4] = {w.x, w.y, w.z, w.w};
+#pragma unroll
+    for (int j = 0; j < 16; ++j) take(static_cast<int8_t>(ws[j / 4] >> (8 * (j % 4))), static_cast<uint32_t>(i) + j);
+  };
+  size_t i = static_cast<size_t>(lane) * 16;
+  for (; i + 3 * kWave * 16 < whole; i += 4 * kWave * 16) {   // four loads in flight per lane, taken in ascending order
+    vuint4 w[4];
+#pragma unroll
+    for (int u = 0; u < 4; ++u) w[u] = __builtin_nontemporal_load(reinterpret_cast<const vuint4*>(p + i + u * kWave * 16));
+#pragma unroll
+    for (int u = 0; u < 4; ++u) take16(w[u], i + u * kWave * 16);
+  }
+  for (; i < whole; i += kWave * 16) take16(*reinterpret_cast<const vuint4*>(p + i), i);
+  for (size_t r = whole + lane; r < len; r += kWave) take(p[r], static_cast<uint32_t>(r));
+  // key: the value in the high word (flipped for a minimum), the complement of the index below it:
+  // the largest key is the best value at the lowest index
+  uint64_t key = (static_cast<uint64_t>(static_cast<uint32_t>(want_max ? best + 129 : 128 - best)) << 32) | (0xFFFFFFFFu - best_at);
+#pragma unroll
+  for (int s = 32; s >= 1; s >>= 1) {
+    const uint32_t hi = __shfl_xor(static_cast<uint32_t>(key >> 32), s), lo = __shfl_xor(static_cast<uint32_t>(key), s);
+    const uint64_t other = (static_cast<uint64_t>(hi) << 32) | lo;
+    key = other > key ? other : key;
+  }
+  if (lane == 0) {
+    const uint32_t at = 0xFFFFFFFFu - static_cast<uint32_t>(key);
+    if (out_i64) static_cast<int64_t*>(out)[row] = static_cast<int64_t>(at);
+    else static_cast<int32_t*>(out)[row] = static_cast<int32_t>(at);
+  }
+}
+
 // q_argmax / q_argmin on the stored integers: per output position, the first index along `dim` of the
 // largest (smallest) value -- ties keep the lowest index, as the reference's fold with a strict
 // comparison does (crates/burn-ndarray/src/ops/base.rs:1727-1750). One thread per output position.
@@ -325,6 +419,54 @@ IndexMap make_index_map(const size_t* out_shape, int rank, const int64_t* stride
   return d;
 }
 
+FastDiv make_fast_div(uint32_t d) {
+  FastDiv f{};
+  f.d = d;
+  uint32_t l = 0;
+  while ((1ull << l) < d) ++l;                       // ceil(log2 d)
+  f.s = 31 + l;
+  f.m = static_cast<uint32_t>(((1ull << f.s) + d - 1) / d);   // ceil(2^(31 + l) / d) <= 2^32 - 1 for d >= 1 ... (d = 1: 2^31)
+  return f;
+}
+
+// Launches the row-run copy when the map allows it; returns false (nothing launched) otherwise.
+// `elem_bits`: bits per element on both sides (8 for native and 8-bit values, 4, 2, or 32 for scales).
+bool try_row_copy(const void* src, void* dst, const size_t* out_shape, int rank, const int64_t* stride, int64_t base, int index_dim,
+                  int index_mode, const void* indices, int index_dtype, size_t index_limit, int elem_bits, hipStream_t st) {
+  if (rank < 1 || stride[rank - 1] != 1 || index_dim == rank - 1 || (index_dim >= 0 && index_mode != 1)) return false;
+  const size_t row_bits = out_shape[rank - 1] * static_cast<size_t>(elem_bits);
+  size_t rows = 1;
+  for (int a = 0; a + 1 < rank; ++a) rows *= out_shape[a];
+  if (rows == 0 || row_bits == 0) return false;
+  auto aligned = [&](size_t vb) {
+    if (row_bits % (8 * vb) != 0 || (base * elem_bits) % static_cast<int64_t>(8 * vb) != 0) return false;
+    for (int a = 0; a + 1 < rank; ++a)
+      if ((stride[a] * elem_bits) % static_cast<int64_t>(8 * vb) != 0) return false;
+    return (reinterpret_cast<uintptr_t>(src) % vb) == 0 && (reinterpret_cast<uintptr_t>(dst) % vb) == 0;
+  };
+  const size_t vb = aligned(16) ? 16 : (aligned(4) ? 4 : 0);
+  if (vb == 0) return false;
+  const size_t per_row = row_bits / (8 * vb), total = rows * per_row;
+  if (total >= 0x7FFFFFFFull || rows >= 0x7FFFFFFFull) return false;
+  RowMap d{};
+  d.rank = rank - 1;
+  for (int a = 0; a + 1 < rank; ++a) {
+    d.div[a] = make_fast_div(static_cast<uint32_t>(out_shape[a]));
+    d.stride[a] = stride[a] * elem_bits / 8;
+  }
+  d.base = base * elem_bits / 8;
+  d.per_row = make_fast_div(static_cast<uint32_t>(per_row));
+  d.index_dim = index_dim;
+  d.index_i64 = index_dtype == BQ_I64;
+  d.index_limit = static_cast<int64_t>(index_limit);
+  dim3 grid(static_cast<unsigned>((total + 255) / 256)), tb(256);
+  const unsigned char* s8 = static_cast<const unsigned char*>(src);
+  unsigned char* d8 = static_cast<unsigned char*>(dst);
+  if (vb == 16) hipLaunchKernelGGL(row_copy_kernel<vuint4>, grid, tb, 0, st, s8, d8, static_cast<uint32_t>(total), d, indices);
+  else hipLaunchKernelGGL(row_copy_kernel<uint32_t>, grid, tb, 0, st, s8, d8, static_cast<uint32_t>(total), d, indices);
+  return true;
+}
+
 }  // namespace
 
 // Values of `out_shape` (every extent below 2^32) gathered through the index map described above.
@@ -335,8 +477,15 @@ bq_status launch_q_index_map(const void* src, void* dst, const size_t* out_shape
   size_t n = 1;
   for (int a = 0; a < rank; ++a) n *= out_shape[a];
   if (n == 0) return BQ_OK;
-  const IndexMap d = make_index_map(out_shape, rank, stride, base, index_dim, index_mode, index_dtype, index_limit);
   const int bits = value_bits(value);
+  // whole rows of bytes when both sides store the values the same way (8-bit values: native bytes are the packed words' bytes)
+  if ((src_native == dst_native || bits == 8) &&
+      try_row_copy(src, dst, out_shape, rank, stride, base, index_dim, index_mode, indices, index_dtype, index_limit,
+                   (src_native && dst_native) ? 8 : bits, st)) {
+    BQ_HIP(hipGetLastError());
+    return BQ_OK;
+  }
+  const IndexMap d = make_index_map(out_shape, rank, stride, base, index_dim, index_mode, index_dtype, index_limit);
   const size_t units = (n + 32 / bits - 1) / (32 / bits);
   if ((units + 255) / 256 > 0x7FFFFFFFu) BQ_FAIL(BQ_ERR_SIZE, "an index map over %zu values exceeds the launch grid", n);
   dim3 grid(static_cast<unsigned>((units + 255) / 256)), tb(256);
@@ -355,6 +504,10 @@ bq_status launch_f32_index_map(const float* src, float* dst, const size_t* out_s
   size_t n = 1;
   for (int a = 0; a < rank; ++a) n *= out_shape[a];
   if (n == 0) return BQ_OK;
+  if (try_row_copy(src, dst, out_shape, rank, stride, base, index_dim, index_mode, indices, index_dtype, index_limit, 32, st)) {
+    BQ_HIP(hipGetLastError());
+    return BQ_OK;
+  }
   const IndexMap d = make_index_map(out_shape, rank, stride, base, index_dim, index_mode, index_dtype, index_limit);
   if ((n + 255) / 256 > 0x7FFFFFFFu) BQ_FAIL(BQ_ERR_SIZE, "an index map over %zu scales exceeds the launch grid", n);
   hipLaunchKernelGGL(f32_index_map_kernel, dim3(static_cast<unsigned>((n + 255) / 256)), dim3(256), 0, st, src, dst, n, d, indices);
@@ -372,6 +525,12 @@ bq_status launch_q_arg(const void* src, int value, bool native, size_t outer, si
   const uint32_t* s32 = static_cast<const uint32_t*>(src);
   const int bits = value_bits(value);
   const bool i64 = out_dtype == BQ_I64;
+  if ((bits == 8 || native) && inner == 1 && len >= 64 && len < 0xFFFFFFFFull && (outer + 3) / 4 <= 0x7FFFFFFFu) {
+    hipLaunchKernelGGL(q8_arg_last_kernel, dim3(static_cast<unsigned>((outer + 3) / 4)), dim3(256), 0, st,
+                       static_cast<const int8_t*>(src), outer, len, want_max, i64, out);
+    BQ_HIP(hipGetLastError());
+    return BQ_OK;
+  }
   if (bits == 8) hipLaunchKernelGGL(q_arg_kernel<8>, grid, tb, 0, st, s32, native, outer, len, inner, want_max, i64, out);
   else if (bits == 4) hipLaunchKernelGGL(q_arg_kernel<4>, grid, tb, 0, st, s32, native, outer, len, inner, want_max, i64, out);
   else hipLaunchKernelGGL(q_arg_kernel<2>, grid, tb, 0, st, s32, native, outer, len, inner, want_max, i64, out);

@@ -43,6 +43,9 @@ namespace {
 #endif
 constexpr int kThreads = BQ_QUANT_THREADS;
 
+// b of QuantValue::range() by values per word: Q8S 127, Q4S 7, Q2S 1
+constexpr float qmax_of(int vpl) { return vpl == 4 ? 127.0f : (vpl == 8 ? 7.0f : 1.0f); }
+
 template <int VPL>
 struct Vals {
   float v[VPL];
@@ -76,7 +79,7 @@ __device__ __forceinline__ float absmax_vals(const Vals<VPL>& a) {
 // FULL: a full-range value (Q8F, Q4F): the lower clamp is -QMAX - 1.
 template <int VPL, bool FULL = false>
 __device__ __forceinline__ uint32_t quantize_pack_div(const Vals<VPL>& a, float s) {
-  constexpr float QMAX = (VPL == 4) ? 127.0f : 7.0f, QMIN = FULL ? -QMAX - 1.0f : -QMAX;
+  constexpr float QMAX = qmax_of(VPL), QMIN = FULL ? -QMAX - 1.0f : -QMAX;
   int q[VPL];
 #pragma unroll
   for (int i = 0; i < VPL; ++i) q[i] = quantize_div(a.v[i], s, QMIN, QMAX);
@@ -89,7 +92,7 @@ __device__ __forceinline__ uint32_t quantize_pack_div(const Vals<VPL>& a, float 
 // (A full-range value always clamps: absmax / s is QMAX + 0.5, which rounds to QMAX + 1.)
 template <int VPL, bool CLAMP, bool FULL = false>
 __device__ __forceinline__ uint32_t quantize_pack_recip(const Vals<VPL>& a, float s, float r) {
-  constexpr float QMAX = (VPL == 4) ? 127.0f : 7.0f, QMIN = FULL ? -QMAX - 1.0f : -QMAX;
+  constexpr float QMAX = qmax_of(VPL), QMIN = FULL ? -QMAX - 1.0f : -QMAX;
   int q[VPL];
 #pragma unroll
   for (int i = 0; i < VPL; ++i) {
@@ -358,10 +361,12 @@ __global__ void __launch_bounds__(kThreads)
 quantize_tensor_kernel(const float* __restrict__ x, size_t n, const float* __restrict__ scale,
                        float* __restrict__ scale_out, uint32_t* __restrict__ out, int sdt) {
   constexpr int U = kTensorUnroll;
-  constexpr float QMAX = (VPL == 4) ? 127.0f : 7.0f, QMIN = FULL ? -QMAX - 1.0f : -QMAX;
+  constexpr float QMAX = qmax_of(VPL), QMIN = FULL ? -QMAX - 1.0f : -QMAX;
   constexpr float SPAN = QMAX - QMIN;
   const size_t words = n / VPL;
-  const size_t piece = piece_back_to_front<pieces_per_chunk<VPL>(kThreads, kTensorUnroll)>(blockIdx.x, gridDim.x);
+  // (2-bit values: a piece of 16 floats per lane and word is as large as two first-pass chunks; plain order)
+  constexpr unsigned PPC = pieces_per_chunk<VPL>(kThreads, kTensorUnroll);
+  const size_t piece = PPC == 0 ? static_cast<size_t>(blockIdx.x) : piece_back_to_front<(PPC == 0 ? 1u : PPC)>(blockIdx.x, gridDim.x);
   const size_t base = piece * (kThreads * U) + threadIdx.x;
   Vals<VPL> a[U];
 #pragma unroll
@@ -653,9 +658,37 @@ __device__ __forceinline__ float workgroup_sum(float v) {
 
 __global__ void __launch_bounds__(kThreads)
 abs_sum_kernel(const float* __restrict__ x, size_t n, float* __restrict__ cells) {
+  // 16-byte loads, four in flight per lane, four independent vector sums per lane (a fixed
+  // function of the element index, so the result repeats run to run); scalar loads when x is not
+  // 16-byte aligned, and for the last n % 4 elements.
   const size_t stride = static_cast<size_t>(gridDim.x) * kThreads;
+  const size_t first = static_cast<size_t>(blockIdx.x) * kThreads + threadIdx.x;
   float sum = 0.0f;
-  for (size_t i = static_cast<size_t>(blockIdx.x) * kThreads + threadIdx.x; i < n; i += stride) sum += fabsf(x[i]);
+  if ((reinterpret_cast<uintptr_t>(x) & 15u) == 0) {
+    const size_t n4 = n / 4;
+    const vfloat4* p = reinterpret_cast<const vfloat4*>(x);
+    vfloat4 acc[4];
+#pragma unroll
+    for (int u = 0; u < 4; ++u) acc[u] = vfloat4{0.f, 0.f, 0.f, 0.f};
+    size_t i = first;
+    for (; i + 3 * stride < n4; i += 4 * stride) {
+      vfloat4 v[4];
+#pragma unroll
+      for (int u = 0; u < 4; ++u) v[u] = __builtin_nontemporal_load(p + i + u * stride);
+#pragma unroll
+      for (int u = 0; u < 4; ++u) acc[u] += vfloat4{fabsf(v[u].x), fabsf(v[u].y), fabsf(v[u].z), fabsf(v[u].w)};
+    }
+    for (; i < n4; i += stride) {
+      const vfloat4 v = __builtin_nontemporal_load(p + i);
+      acc[0] += vfloat4{fabsf(v.x), fabsf(v.y), fabsf(v.z), fabsf(v.w)};
+    }
+    const vfloat4 a = (acc[0] + acc[1]) + (acc[2] + acc[3]);
+    sum = (a.x + a.y) + (a.z + a.w);
+    if (first == 0)
+      for (size_t r = n4 * 4; r < n; ++r) sum += fabsf(x[r]);
+  } else {
+    for (size_t i = first; i < n; i += stride) sum += fabsf(x[i]);
+  }
   const float total = workgroup_sum(sum);
   if (threadIdx.x == 0) cells[blockIdx.x] = total;
 }
@@ -1001,7 +1034,8 @@ extern "C" bq_status bqk_scales_from_absmax(const float* absmax, size_t n, int32
 }
 
 static bq_status check_value_store(int32_t value, int32_t store, size_t n) {
-  if (!value_known(value)) BQ_FAIL(BQ_ERR_UNSUPPORTED_SCHEME, "unknown quant value %d", value);
+  // (2-bit values: the per-tensor kernel takes them packed; the block kernels do not)
+  if (!value_supported(value)) BQ_FAIL(BQ_ERR_UNSUPPORTED_SCHEME, "unknown quant value %d", value);
   if (store == BQ_STORE_NATIVE) {
     if (value_bits(value) != 8)
       BQ_FAIL(BQ_ERR_UNSUPPORTED_SCHEME, "Can't store native sub-byte values");
@@ -1039,7 +1073,10 @@ static bq_status quantize_per_tensor_impl(const float* x, size_t n, const float*
   const size_t per_wg = static_cast<size_t>(kThreads) * kTensorUnroll;
   size_t g = (n / vpl + per_wg - 1) / per_wg;
   if (g < 1) g = 1;
-  g = eight ? grid_back_to_front<pieces_per_chunk<4>(kThreads, kTensorUnroll)>(g) : grid_back_to_front<pieces_per_chunk<8>(kThreads, kTensorUnroll)>(g);
+  const int bits = value_bits(value);
+  if (bits == 2 && store != BQ_STORE_PACKED_U32) BQ_FAIL(BQ_ERR_UNSUPPORTED_SCHEME, "2-bit values are quantized per tensor as packed words only");
+  if (bits != 2)
+    g = eight ? grid_back_to_front<pieces_per_chunk<4>(kThreads, kTensorUnroll)>(g) : grid_back_to_front<pieces_per_chunk<8>(kThreads, kTensorUnroll)>(g);
   if (g > 0x7FFFFFFFull) BQ_FAIL(BQ_ERR_SIZE, "quantize of %zu values exceeds the launch grid", n);
   dim3 grid(static_cast<unsigned>(g)), tb(kThreads);
   uint32_t* out = static_cast<uint32_t*>(values);
@@ -1047,6 +1084,9 @@ static bq_status quantize_per_tensor_impl(const float* x, size_t n, const float*
   if (eight) {
     if (from_absmax) { if (full) BQ_TENSOR(4, true, true); else BQ_TENSOR(4, true, false); }
     else { if (full) BQ_TENSOR(4, false, true); else BQ_TENSOR(4, false, false); }
+  } else if (bits == 2) {
+    if (from_absmax) { if (full) BQ_TENSOR(16, true, true); else BQ_TENSOR(16, true, false); }
+    else { if (full) BQ_TENSOR(16, false, true); else BQ_TENSOR(16, false, false); }
   } else {
     if (from_absmax) { if (full) BQ_TENSOR(8, true, true); else BQ_TENSOR(8, true, false); }
     else { if (full) BQ_TENSOR(8, false, true); else BQ_TENSOR(8, false, false); }

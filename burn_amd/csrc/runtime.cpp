@@ -1005,6 +1005,12 @@ static bq_status quantize_pass(const bq_tensor* x, const bq_scheme* scheme, bq_t
         if (rc == BQ_OK) rc = launch_scale_from_cells(cells, scheme->value, sdt, q->scales(), st);
         if (rc != BQ_OK) break;
       }
+      if (per_tensor && value_bits(scheme->value) == 2 && scheme->store == BQ_STORE_PACKED_U32 &&
+          (reinterpret_cast<uintptr_t>(xin) & 15u) == 0) {
+        // a per-tensor 2-bit quantize (a BitNet weight): the streaming per-tensor kernel, 16 values per word
+        rc = launch_quantize_per_tensor(xin, n, q->scales(), false, nullptr, scheme->value, scheme->store, q->data, sdt, st);
+        break;
+      }
       size_t blk[BQ_MAX_RANK];
       block_dims(*scheme, x->rank, blk);
       rc = launch_quantize_rect(xin, x->shape, x->rank, per_tensor ? nullptr : blk, scheme->value, scheme->store,
