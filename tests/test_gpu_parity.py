@@ -1750,6 +1750,111 @@ def test_integer_domain_ops_against_numpy(dev, value, store):
     assert (q == np.take(q_ref, [0, 0, 7, 7], axis=1)).all()
 
 
+def test_integer_domain_ops_random_configurations(dev):
+    """Seeded draws over ranks 1-4, Q8S / Q4S / Q2S, packed and native stores, per-tensor schemes and blocks
+    along the last dim: random slices (negative indices, steps of either sign, single indices), selects,
+    expands and arg reductions against numpy on the oracle's integers and scales. Both routes of the
+    index map run: whole-row copies where the last dim is kept or cut at word boundaries, the element
+    gather elsewhere."""
+    rng = np.random.default_rng(20260)
+    done = {"slice": 0, "select": 0, "expand": 0, "arg": 0, "declined": 0}
+    for case in range(160):
+        value = [QuantValue.Q8S, QuantValue.Q4S, QuantValue.Q2S][case % 3]
+        store = QuantStore.PackedU32 if (case // 3) % 2 == 0 else QuantStore.Native
+        nq = {QuantValue.Q8S: 4, QuantValue.Q4S: 8, QuantValue.Q2S: 16}[value]
+        rank = int(rng.integers(1, 5))
+        last = int(rng.choice([32, 64, 96, 128]))
+        shape = tuple(int(rng.integers(1, 7)) for _ in range(rank - 1)) + (last,)
+        blocked = case % 4 == 1
+        scheme = QuantScheme(value=value, store=store)
+        if blocked:
+            scheme = scheme.per_block((32,))
+        x = awkward(shape, 9000 + case)
+        tq = QTensorOps.quantize_dynamic(FloatOps.float_from_data(x, dev), scheme)
+        q_ref, s_ref = co.quantize_dynamic(x, oscheme(scheme))
+        pshape = shape[:-1] + (last // 32,) if blocked else None
+        s_nd = s_ref.reshape(pshape) if blocked else None
+
+        def check(t, q_want, s_want):
+            q, s = unpack_blob(QTensorOps.q_into_data(t))
+            assert t.shape == q_want.shape, (case, t.shape, q_want.shape)
+            assert (q == q_want).all(), case
+            assert s.reshape(-1).tobytes() == np.ascontiguousarray(s_want, np.float32).reshape(-1).tobytes(), case
+
+        kind = case % 5
+        if kind in (0, 1):          # slice: any cut of the leading dims; the last dim in whole blocks / words, or freely
+            slices = []
+            for a, n in enumerate(shape[:-1]):
+                pick = int(rng.integers(0, 4))
+                if pick == 0:
+                    slices.append(slice(None))
+                elif pick == 1:
+                    slices.append(int(rng.integers(-n, n)))
+                else:
+                    lo, hi = sorted(int(v) for v in rng.integers(-n, n + 1, 2))
+                    step = int(rng.choice([1, 1, 2, -1, -2]))
+                    slices.append(slice(lo, hi if hi != lo else None, step))
+            free = kind == 1 and not blocked and (value == QuantValue.Q8S or store == QuantStore.Native)
+            if free:                # any range and step: the result may not fill packed words (Q8S goes native)
+                lo, hi = sorted(int(v) for v in rng.integers(0, last + 1, 2))
+                slices.append(slice(lo, max(hi, lo + 1), int(rng.choice([1, 3, -1]))))
+            else:
+                lo = 32 * int(rng.integers(0, last // 32))
+                hi = 32 * int(rng.integers(lo // 32 + 1, last // 32 + 1))
+                slices.append(slice(lo, hi))
+            want_q = burn_slice(q_ref, slices)
+            if want_q.size == 0:
+                continue
+            if blocked:
+                sb = list(slices[:-1]) + [slice(slices[-1].start // 32, slices[-1].stop // 32)]
+                want_s = burn_slice(s_nd, sb)
+            else:
+                want_s = s_ref
+            check(QTensorOps.q_slice(tq, tuple(slices)), want_q, want_s)
+            done["slice"] += 1
+        elif kind == 2:             # select along a leading dim (blocks of 1 there); the last dim only per tensor
+            dim = int(rng.integers(0, rank)) if not blocked else int(rng.integers(0, max(rank - 1, 1)))
+            if blocked and rank == 1:
+                with pytest.raises(ba.BurnqError):
+                    QTensorOps.q_select(tq, 0, IntOps.int_from_data(np.int64([0]), dev))
+                done["declined"] += 1
+                continue
+            count = int(rng.integers(1, 9)) if dim < rank - 1 else nq * int(rng.integers(1, 4))
+            idx = rng.integers(0, shape[dim], count)
+            it = IntOps.int_from_data(idx.astype(np.int32 if case % 2 else np.int64), dev)
+            if dim == rank - 1 and store == QuantStore.PackedU32 and value != QuantValue.Q8S and count % nq:
+                continue
+            want_s = np.take(s_nd, idx, axis=dim) if blocked else s_ref
+            check(QTensorOps.q_select(tq, dim, it), np.take(q_ref, idx, axis=dim), want_s)
+            done["select"] += 1
+        elif kind == 3:             # expand: new leading dims and dims of 1
+            if rank > 1 and shape[0] != 1:
+                src_t, src_q, src_s = QTensorOps.q_slice(tq, (0,)), q_ref[0:1], (s_nd[0:1] if blocked else s_ref)
+            else:
+                src_t, src_q, src_s = tq, q_ref, (s_nd if blocked else s_ref)
+            lead = tuple(int(v) for v in rng.integers(1, 4, int(rng.integers(0, 3))))
+            target = lead + ((int(rng.integers(2, 5)),) + src_q.shape[1:] if rank > 1 else src_q.shape)
+            if len(target) > 6:
+                continue
+            want_s = np.broadcast_to(src_s, lead + ((target[len(lead)],) + src_s.shape[1:] if rank > 1 else src_s.shape)) if blocked else s_ref
+            check(QTensorOps.q_expand(src_t, target), np.broadcast_to(src_q, target), want_s)
+            done["expand"] += 1
+        else:                       # arg reductions: per tensor along any dim
+            if blocked:             # blocks of 32 along a longer last dim: the order of the integers is not the values'
+                if last > 32:
+                    with pytest.raises(ba.BurnqError) as e:
+                        QTensorOps.q_argmax(tq, rank - 1)
+                    assert e.value.status == ba._lib.ERR_UNSUPPORTED_OP
+                    done["declined"] += 1
+                continue
+            dim = int(rng.integers(0, rank))
+            for fn, npf in ((QTensorOps.q_argmax, np.argmax), (QTensorOps.q_argmin, np.argmin)):
+                got = IntOps.int_into_data(fn(tq, dim, ba.I32 if case % 2 else ba.I64))
+                assert (got == np.expand_dims(npf(q_ref, axis=dim), dim)).all(), (case, dim)
+            done["arg"] += 1
+    assert done["slice"] >= 40 and done["select"] >= 15 and done["expand"] >= 15 and done["arg"] >= 15, done
+
+
 def _int8(dev, floats):
     """The reference tests' QTensor::int8: quantize_dynamic, Q8S per tensor (native store, as the backends
     that run them; crates/burn-backend-tests/tests/tensor/float/quantization/mod.rs:23-50)."""
