@@ -31,6 +31,27 @@ def test_library_exports_every_declared_symbol():
     assert sorted(_lib.SIGNATURES) == names
 
 
+def test_entry_points_named_in_the_guides_exist():
+    """Every bq_* / bqk_* function the written guides name (binding guide, design notes, readme) is one
+    the header declares: a maintainer who binds from the text gets names that link."""
+    exported = set(declared_symbols())
+    types = {"bq_status", "bq_tensor", "bq_device", "bq_scheme", "bq_graph", "bq_pack", "bq_pack_writer", "bq_pack_entry",
+             "bq_backend", "bq_oracle"}          # C types, the oracle's file stem, and one name the text says was not built
+    unknown = {}
+    for doc in ("INTEGRATION.md", "DESIGN.md", "README.md"):
+        path = os.path.join(ROOT, doc)
+        if not os.path.exists(path):
+            continue
+        for name in set(re.findall(r"\b(bqk?_[a-z0-9_]*[a-z0-9])\b(?![_*])", open(path).read())):
+            if name in exported or name in types:
+                continue
+            # families written with a wildcard or a brace list (bq_pack_*, bq_graph_{begin,end}_capture) leave a prefix
+            if any(e.startswith(name + "_") for e in exported):
+                continue
+            unknown.setdefault(doc, []).append(name)
+    assert not unknown, unknown
+
+
 def test_scheme_struct_layout_matches_header():
     assert C.sizeof(_lib.CScheme) == 16
     c = QuantScheme(QuantValue.Q4S, (32,), QuantStore.PackedU32).to_c()
