@@ -219,8 +219,16 @@ bq_status launch_f32_gather(const float* src, float* dst, const size_t* src_shap
 // reference panics on, is clamped into it: never a fault.
 namespace {
 
+struct FastDiv {
+  uint32_t m, s, d;
+};
+__device__ __forceinline__ uint32_t fast_div(uint32_t n, const FastDiv& f) {
+  return static_cast<uint32_t>((static_cast<uint64_t>(n) * f.m) >> f.s);
+}
 struct IndexMap {
   int rank;
+  int fast;                      // every element index is below 2^31: `div` holds the constants for the output extents
+  FastDiv div[BQ_MAX_RANK];
   uint32_t shape[BQ_MAX_RANK];   // output shape
   int64_t stride[BQ_MAX_RANK];   // source elements per step of output dim a
   int64_t base;
@@ -233,9 +241,17 @@ struct IndexMap {
 __device__ __forceinline__ int64_t mapped_index(const IndexMap& d, size_t e, const void* __restrict__ indices) {
   int64_t idx = d.base;
   size_t rem = e;
+  uint32_t rem32 = static_cast<uint32_t>(e);
   for (int a = d.rank - 1; a >= 0; --a) {
-    const size_t c = rem % d.shape[a];
-    rem /= d.shape[a];
+    size_t c;
+    if (d.fast) {  // (uniform over the launch)
+      const uint32_t q = fast_div(rem32, d.div[a]);
+      c = rem32 - q * d.div[a].d;
+      rem32 = q;
+    } else {
+      c = rem % d.shape[a];
+      rem /= d.shape[a];
+    }
     int64_t i = static_cast<int64_t>(c);
     if (a == d.index_dim) {
       const size_t at = d.index_mode == 2 ? e : c;
@@ -287,12 +303,6 @@ f32_index_map_kernel(const float* __restrict__ src, float* __restrict__ dst, siz
 // leaves the last dim alone, or cuts it at word boundaries). A lane copies 16 (or 4) bytes; the
 // row's coordinates come from divisions by constants the host prepared (q = (n * m) >> s, exact for
 // n < 2^31), a few instructions per dim instead of a 64-bit division each.
-struct FastDiv {
-  uint32_t m, s, d;
-};
-__device__ __forceinline__ uint32_t fast_div(uint32_t n, const FastDiv& f) {
-  return static_cast<uint32_t>((static_cast<uint64_t>(n) * f.m) >> f.s);
-}
 struct RowMap {
   int rank;                        // outer dims (output rank - 1)
   FastDiv div[BQ_MAX_RANK];        // by the extent of outer dim a
@@ -403,22 +413,6 @@ q_arg_kernel(const uint32_t* __restrict__ src, bool native, size_t outer, size_t
   else static_cast<int32_t*>(out)[pos] = static_cast<int32_t>(best_at);
 }
 
-IndexMap make_index_map(const size_t* out_shape, int rank, const int64_t* stride, int64_t base, int index_dim, int index_mode,
-                        int index_dtype, size_t index_limit) {
-  IndexMap d{};
-  d.rank = rank;
-  for (int a = 0; a < rank; ++a) {
-    d.shape[a] = static_cast<uint32_t>(out_shape[a]);
-    d.stride[a] = stride[a];
-  }
-  d.base = base;
-  d.index_dim = index_dim;
-  d.index_mode = index_mode;
-  d.index_i64 = index_dtype == BQ_I64;
-  d.index_limit = static_cast<int64_t>(index_limit);
-  return d;
-}
-
 FastDiv make_fast_div(uint32_t d) {
   FastDiv f{};
   f.d = d;
@@ -427,6 +421,26 @@ FastDiv make_fast_div(uint32_t d) {
   f.s = 31 + l;
   f.m = static_cast<uint32_t>(((1ull << f.s) + d - 1) / d);   // ceil(2^(31 + l) / d) <= 2^32 - 1 for d >= 1 ... (d = 1: 2^31)
   return f;
+}
+
+IndexMap make_index_map(const size_t* out_shape, int rank, const int64_t* stride, int64_t base, int index_dim, int index_mode,
+                        int index_dtype, size_t index_limit) {
+  IndexMap d{};
+  d.rank = rank;
+  size_t n = 1;
+  for (int a = 0; a < rank; ++a) {
+    d.shape[a] = static_cast<uint32_t>(out_shape[a]);
+    d.stride[a] = stride[a];
+    d.div[a] = make_fast_div(static_cast<uint32_t>(out_shape[a] ? out_shape[a] : 1));
+    n *= out_shape[a];
+  }
+  d.fast = n < 0x7FFFFFFFull;
+  d.base = base;
+  d.index_dim = index_dim;
+  d.index_mode = index_mode;
+  d.index_i64 = index_dtype == BQ_I64;
+  d.index_limit = static_cast<int64_t>(index_limit);
+  return d;
 }
 
 // Launches the row-run copy when the map allows it; returns false (nothing launched) otherwise.
