@@ -1750,7 +1750,7 @@ extern "C" bq_status bq_q_slice(const bq_tensor* t, const int64_t* starts, const
     int64_t start = 0, end = size, step = 1;
     if (a < n_slices) {
       step = steps[a];
-      if (step == 0) BQ_FAIL(BQ_ERR_SHAPE, "Step cannot be zero");
+      if (step == 0 || step == INT64_MIN) BQ_FAIL(BQ_ERR_SHAPE, "Step cannot be zero");  // (INT64_MIN has no magnitude)
       start = signed_index(starts[a], size);
       end = ends[a] == INT64_MAX ? size : signed_index(ends[a], size);   // INT64_MAX: to the end of the dim
     }
