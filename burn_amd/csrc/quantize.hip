@@ -411,6 +411,44 @@ quantize_tensor_kernel(const float* __restrict__ x, size_t n, const float* __res
   }
 }
 
+// 2-bit values against a given scale: 16 values to the word, so a lane that owned a whole word would
+// read 64 bytes at a stride of 64 (the per-tensor kernel above does, at 3.6 TB/s). Here a lane takes
+// one 16-byte piece per load, consecutive lanes consecutive pieces: the four lanes of a quad hold the
+// four quarters of a word, put their bytes together with two DPP swaps, and lane i of the quad keeps
+// the word of load i. n is a multiple of 16, x 16-byte aligned.
+__global__ void __launch_bounds__(256)
+quantize_tensor_2bit_kernel(const float* __restrict__ x, size_t n, const float* __restrict__ scale, float qmin,
+                            uint32_t* __restrict__ out) {
+  const float s = valid_scale(scale[0]);
+  const bool fast = recip_path_ok(s);
+  const float r = recip_exact(s);
+  const size_t pieces = n / 4, first = static_cast<size_t>(blockIdx.x) * 1024 + threadIdx.x;
+  vfloat4 v[4];
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const size_t f = first + static_cast<size_t>(i) * 256;
+    v[i] = f < pieces ? __builtin_nontemporal_load(reinterpret_cast<const vfloat4*>(x) + f) : vfloat4{0.f, 0.f, 0.f, 0.f};
+  }
+  uint32_t mine = 0;
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const float e[4] = {v[i].x, v[i].y, v[i].z, v[i].w};
+    uint32_t b = 0;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const int q = fast ? quantize_recip(e[j], s, r, qmin, 1.0f) : quantize_div(e[j], s, qmin, 1.0f);
+      b |= (static_cast<uint32_t>(q) & 3u) << (2 * j);
+    }
+    uint32_t w = b << (8u * (threadIdx.x & 3u));
+    w |= static_cast<uint32_t>(__builtin_amdgcn_update_dpp(0, static_cast<int>(w), 0xB1, 0xF, 0xF, false));  // lanes 2p <-> 2p + 1
+    w |= static_cast<uint32_t>(__builtin_amdgcn_update_dpp(0, static_cast<int>(w), 0x4E, 0xF, 0xF, false));  // pairs of a quad
+    if ((threadIdx.x & 3u) == static_cast<unsigned>(i)) mine = w;
+  }
+  // load i of this quad was word 64 i + tid / 4 of the workgroup's 256
+  const size_t word = static_cast<size_t>(blockIdx.x) * 256 + (threadIdx.x & 3u) * 64u + threadIdx.x / 4u;
+  if (word * 16 < n) __builtin_nontemporal_store(mine, out + word);
+}
+
 // Unaligned input pointer: one value per lane, byte stores (native Q8S only).
 __global__ void __launch_bounds__(kThreads)
 quantize_tensor_scalar_kernel(const float* __restrict__ x, size_t n,
@@ -1084,6 +1122,9 @@ static bq_status quantize_per_tensor_impl(const float* x, size_t n, const float*
   if (eight) {
     if (from_absmax) { if (full) BQ_TENSOR(4, true, true); else BQ_TENSOR(4, true, false); }
     else { if (full) BQ_TENSOR(4, false, true); else BQ_TENSOR(4, false, false); }
+  } else if (bits == 2 && !from_absmax && n / 4 + 1023 < 0x7FFFFFFFull * 1024ull) {
+    hipLaunchKernelGGL(quantize_tensor_2bit_kernel, dim3(static_cast<unsigned>((n / 4 + 1023) / 1024)), dim3(256), 0, st, x, n, scale,
+                       static_cast<float>(value_qmin(value)), out);
   } else if (bits == 2) {
     if (from_absmax) { if (full) BQ_TENSOR(16, true, true); else BQ_TENSOR(16, true, false); }
     else { if (full) BQ_TENSOR(16, false, true); else BQ_TENSOR(16, false, false); }
