@@ -213,6 +213,10 @@ bq_status launch_q_index_map(const void* src, void* dst, const size_t* out_shape
 bq_status launch_f32_index_map(const float* src, float* dst, const size_t* out_shape, int rank, const int64_t* stride, int64_t base,
                                int index_dim, int index_mode, const void* indices, int index_dtype, size_t index_limit,
                                hipStream_t stream);
+bq_status launch_index_map_pair(const void* src, void* dst, const size_t* out_shape, const int64_t* stride, int64_t base, int value,
+                                bool src_native, bool dst_native, const float* s_src, float* s_dst, const size_t* s_shape,
+                                const int64_t* s_stride, int64_t s_base, int rank, int index_dim, int index_mode, const void* indices,
+                                int index_dtype, size_t index_limit, bool* fused, hipStream_t stream);
 bq_status launch_q_arg(const void* src, int value, bool native, size_t outer, size_t len, size_t inner, bool want_max, int out_dtype,
                        void* out, hipStream_t stream);
 // out[r][c] += bias[c] (out f32 or bf16, in place), and a bf16 -> f32 copy (qmatmul.hip).

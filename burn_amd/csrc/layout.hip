@@ -315,11 +315,8 @@ struct RowMap {
 };
 
 template <typename V>
-__global__ void __launch_bounds__(256)
-row_copy_kernel(const unsigned char* __restrict__ src, unsigned char* __restrict__ dst, uint32_t total, RowMap d,
-                const void* __restrict__ indices) {
-  const uint32_t u = blockIdx.x * 256u + threadIdx.x;
-  if (u >= total) return;
+__device__ __forceinline__ void row_copy_one(const unsigned char* __restrict__ src, unsigned char* __restrict__ dst, uint32_t u,
+                                             const RowMap& d, const void* __restrict__ indices) {
   const uint32_t row = fast_div(u, d.per_row), v = u - row * d.per_row.d;
   int64_t off = d.base + static_cast<int64_t>(v) * static_cast<int64_t>(sizeof(V));
   uint32_t rem = row;
@@ -335,6 +332,40 @@ row_copy_kernel(const unsigned char* __restrict__ src, unsigned char* __restrict
   }
   const V val = __builtin_nontemporal_load(reinterpret_cast<const V*>(src + off));
   __builtin_nontemporal_store(val, reinterpret_cast<V*>(dst) + u);
+}
+
+template <typename V>
+__global__ void __launch_bounds__(256)
+row_copy_kernel(const unsigned char* __restrict__ src, unsigned char* __restrict__ dst, uint32_t total, RowMap d,
+                const void* __restrict__ indices) {
+  const uint32_t u = blockIdx.x * 256u + threadIdx.x;
+  if (u < total) row_copy_one<V>(src, dst, u, d, indices);
+}
+
+// Values and block scales of one op in one launch: the first `blocks_a` workgroups move job a, the
+// rest job b (a second launch for a few megabytes of scales costs more than it moves).
+struct RowJob {
+  const unsigned char* src;
+  unsigned char* dst;
+  uint32_t total;
+  uint32_t wide;  // 16 bytes per lane (else 4)
+  RowMap d;
+};
+
+__global__ void __launch_bounds__(256)
+row_copy_pair_kernel(RowJob a, RowJob b, uint32_t blocks_a, const void* __restrict__ indices) {
+  // (two spelled-out branches: picking one of the two argument structs through a reference would copy both to scratch)
+  if (blockIdx.x < blocks_a) {
+    const uint32_t u = blockIdx.x * 256u + threadIdx.x;
+    if (u >= a.total) return;
+    if (a.wide) row_copy_one<vuint4>(a.src, a.dst, u, a.d, indices);
+    else row_copy_one<uint32_t>(a.src, a.dst, u, a.d, indices);
+  } else {
+    const uint32_t u = (blockIdx.x - blocks_a) * 256u + threadIdx.x;
+    if (u >= b.total) return;
+    if (b.wide) row_copy_one<vuint4>(b.src, b.dst, u, b.d, indices);
+    else row_copy_one<uint32_t>(b.src, b.dst, u, b.d, indices);
+  }
 }
 
 // Arg max / min along the last dim of 8-bit values: a wave per row. A lane walks the row 16 bytes at
@@ -443,10 +474,10 @@ IndexMap make_index_map(const size_t* out_shape, int rank, const int64_t* stride
   return d;
 }
 
-// Launches the row-run copy when the map allows it; returns false (nothing launched) otherwise.
+// Plans the row-run copy when the map allows it; returns false otherwise.
 // `elem_bits`: bits per element on both sides (8 for native and 8-bit values, 4, 2, or 32 for scales).
-bool try_row_copy(const void* src, void* dst, const size_t* out_shape, int rank, const int64_t* stride, int64_t base, int index_dim,
-                  int index_mode, const void* indices, int index_dtype, size_t index_limit, int elem_bits, hipStream_t st) {
+bool plan_row_copy(const void* src, void* dst, const size_t* out_shape, int rank, const int64_t* stride, int64_t base, int index_dim,
+                   int index_mode, int index_dtype, size_t index_limit, int elem_bits, RowJob* job) {
   if (rank < 1 || stride[rank - 1] != 1 || index_dim == rank - 1 || (index_dim >= 0 && index_mode != 1)) return false;
   const size_t row_bits = out_shape[rank - 1] * static_cast<size_t>(elem_bits);
   size_t rows = 1;
@@ -462,7 +493,8 @@ bool try_row_copy(const void* src, void* dst, const size_t* out_shape, int rank,
   if (vb == 0) return false;
   const size_t per_row = row_bits / (8 * vb), total = rows * per_row;
   if (total >= 0x7FFFFFFFull || rows >= 0x7FFFFFFFull) return false;
-  RowMap d{};
+  RowMap& d = job->d;
+  d = RowMap{};
   d.rank = rank - 1;
   for (int a = 0; a + 1 < rank; ++a) {
     d.div[a] = make_fast_div(static_cast<uint32_t>(out_shape[a]));
@@ -473,11 +505,21 @@ bool try_row_copy(const void* src, void* dst, const size_t* out_shape, int rank,
   d.index_dim = index_dim;
   d.index_i64 = index_dtype == BQ_I64;
   d.index_limit = static_cast<int64_t>(index_limit);
-  dim3 grid(static_cast<unsigned>((total + 255) / 256)), tb(256);
-  const unsigned char* s8 = static_cast<const unsigned char*>(src);
-  unsigned char* d8 = static_cast<unsigned char*>(dst);
-  if (vb == 16) hipLaunchKernelGGL(row_copy_kernel<vuint4>, grid, tb, 0, st, s8, d8, static_cast<uint32_t>(total), d, indices);
-  else hipLaunchKernelGGL(row_copy_kernel<uint32_t>, grid, tb, 0, st, s8, d8, static_cast<uint32_t>(total), d, indices);
+  job->src = static_cast<const unsigned char*>(src);
+  job->dst = static_cast<unsigned char*>(dst);
+  job->total = static_cast<uint32_t>(total);
+  job->wide = vb == 16;
+  return true;
+}
+
+// Launches the row-run copy when the map allows it; returns false (nothing launched) otherwise.
+bool try_row_copy(const void* src, void* dst, const size_t* out_shape, int rank, const int64_t* stride, int64_t base, int index_dim,
+                  int index_mode, const void* indices, int index_dtype, size_t index_limit, int elem_bits, hipStream_t st) {
+  RowJob j{};
+  if (!plan_row_copy(src, dst, out_shape, rank, stride, base, index_dim, index_mode, index_dtype, index_limit, elem_bits, &j)) return false;
+  dim3 grid((j.total + 255u) / 256u), tb(256);
+  if (j.wide) hipLaunchKernelGGL(row_copy_kernel<vuint4>, grid, tb, 0, st, j.src, j.dst, j.total, j.d, indices);
+  else hipLaunchKernelGGL(row_copy_kernel<uint32_t>, grid, tb, 0, st, j.src, j.dst, j.total, j.d, indices);
   return true;
 }
 
@@ -526,6 +568,27 @@ bq_status launch_f32_index_map(const float* src, float* dst, const size_t* out_s
   if ((n + 255) / 256 > 0x7FFFFFFFu) BQ_FAIL(BQ_ERR_SIZE, "an index map over %zu scales exceeds the launch grid", n);
   hipLaunchKernelGGL(f32_index_map_kernel, dim3(static_cast<unsigned>((n + 255) / 256)), dim3(256), 0, st, src, dst, n, d, indices);
   BQ_HIP(hipGetLastError());
+  return BQ_OK;
+}
+
+// Values and f32 block scales of one op together, when both maps are whole-row copies: one launch,
+// *fused set. Otherwise nothing is launched and the caller runs the two maps one after the other.
+bq_status launch_index_map_pair(const void* src, void* dst, const size_t* out_shape, const int64_t* stride, int64_t base, int value,
+                                bool src_native, bool dst_native, const float* s_src, float* s_dst, const size_t* s_shape,
+                                const int64_t* s_stride, int64_t s_base, int rank, int index_dim, int index_mode, const void* indices,
+                                int index_dtype, size_t index_limit, bool* fused, hipStream_t st) {
+  *fused = false;
+  const int bits = value_bits(value);
+  if (!(src_native == dst_native || bits == 8)) return BQ_OK;
+  RowJob a{}, b{};
+  if (!plan_row_copy(src, dst, out_shape, rank, stride, base, index_dim, index_mode, index_dtype, index_limit,
+                     (src_native && dst_native) ? 8 : bits, &a) ||
+      !plan_row_copy(s_src, s_dst, s_shape, rank, s_stride, s_base, index_dim, index_mode, index_dtype, index_limit, 32, &b))
+    return BQ_OK;
+  const uint32_t blocks_a = (a.total + 255u) / 256u, blocks_b = (b.total + 255u) / 256u;
+  hipLaunchKernelGGL(row_copy_pair_kernel, dim3(blocks_a + blocks_b), dim3(256), 0, st, a, b, blocks_a, indices);
+  BQ_HIP(hipGetLastError());
+  *fused = true;
   return BQ_OK;
 }
 

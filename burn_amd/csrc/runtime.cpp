@@ -1677,11 +1677,19 @@ static bq_status index_map_impl(const bq_tensor* t, const IndexPlan& p, bq_tenso
   hipStream_t st = t->dev->stream;
   const void* idx = p.indices ? p.indices->data : nullptr;
   const int idx_dtype = p.indices ? p.indices->dtype : BQ_I32;
-  bq_status rc = launch_q_index_map(t->data, q->data, p.out_shape, p.rank, p.stride, p.base, p.index_dim, p.index_mode, idx, idx_dtype,
-                                    p.index_limit, stored_value(t->scheme.value, t->scheme.store), t->scheme.store == BQ_STORE_NATIVE,
-                                    scheme.store == BQ_STORE_NATIVE, st);
+  bq_status rc = BQ_OK;
+  bool fused = false;  // values and block scales in one launch where both are whole-row copies
+  if (scheme.level == BQ_LEVEL_BLOCK)
+    rc = launch_index_map_pair(t->data, q->data, p.out_shape, p.stride, p.base, stored_value(t->scheme.value, t->scheme.store),
+                               t->scheme.store == BQ_STORE_NATIVE, scheme.store == BQ_STORE_NATIVE, t->scales(), q->scales(), p.p_shape,
+                               p.p_stride, p.p_base, p.rank, p.index_dim, p.index_mode, idx, idx_dtype, p.index_limit, &fused, st);
+  if (rc == BQ_OK && !fused)
+    rc = launch_q_index_map(t->data, q->data, p.out_shape, p.rank, p.stride, p.base, p.index_dim, p.index_mode, idx, idx_dtype,
+                            p.index_limit, stored_value(t->scheme.value, t->scheme.store), t->scheme.store == BQ_STORE_NATIVE,
+                            scheme.store == BQ_STORE_NATIVE, st);
   if (rc == BQ_OK && scheme.level == BQ_LEVEL_BLOCK) {
-    rc = launch_f32_index_map(t->scales(), q->scales(), p.p_shape, p.rank, p.p_stride, p.p_base, p.index_dim, p.index_mode, idx, idx_dtype,
+    if (!fused)
+      rc = launch_f32_index_map(t->scales(), q->scales(), p.p_shape, p.rank, p.p_stride, p.p_base, p.index_dim, p.index_mode, idx, idx_dtype,
                               p.index_limit, st);
     if (rc == BQ_OK && scheme.tensor_scale)
       rc = launch_f32_index_map(t->wire_scales(), q->wire_scales(), p.p_shape, p.rank, p.p_stride, p.p_base, p.index_dim, p.index_mode, idx,
