@@ -368,6 +368,13 @@ row_copy_pair_kernel(RowJob a, RowJob b, uint32_t blocks_a, const void* __restri
   }
 }
 
+__device__ __forceinline__ uint32_t pk_max_u16(uint32_t a, uint32_t b) {
+  typedef unsigned short ushort2v __attribute__((ext_vector_type(2)));
+  const ushort2v x = __builtin_bit_cast(ushort2v, a), y = __builtin_bit_cast(ushort2v, b);
+  const ushort2v r = {static_cast<unsigned short>(x.x > y.x ? x.x : y.x), static_cast<unsigned short>(x.y > y.y ? x.y : y.y)};
+  return __builtin_bit_cast(uint32_t, r);
+}
+
 // Arg max / min along the last dim of 8-bit values: a wave per row. A lane walks the row 16 bytes at
 // a time keeping its first best; the wave then takes the best of 64 (value, then lowest index) keys.
 __global__ void __launch_bounds__(256)
@@ -386,10 +393,27 @@ q8_arg_last_kernel(const int8_t* __restrict__ src, size_t rows, size_t len, bool
   };
   const bool vec = (reinterpret_cast<uintptr_t>(p) & 15u) == 0;
   const size_t whole = vec ? len / 16 * 16 : 0;
+  // Sixteen values at a time without a compare per value: a byte u (the value with its sign bit
+  // flipped: unsigned order is the signed order; all bits flipped for a minimum) becomes the 16-bit key
+  // u << 8 | 15 - position, two keys to a register (one byte permute against a constant of position
+  // codes), and packed 16-bit maxima leave the largest value at its lowest position.
+  const uint32_t flip = want_max ? 0x80808080u : 0x7F7F7F7Fu;
   auto take16 = [&](const vuint4& w, size_t i) {
-    const uint32_t ws[4] = {w.x, w.y, w.z, w.w};
+    const uint32_t ws[4] = {w.x ^ flip, w.y ^ flip, w.z ^ flip, w.w ^ flip};
+    uint32_t m = 0;
 #pragma unroll
-    for (int j = 0; j < 16; ++j) take(static_cast<int8_t>(ws[j / 4] >> (8 * (j % 4))), static_cast<uint32_t>(i) + j);
+    for (int q = 0; q < 4; ++q) {
+      // position codes 15 - (4 q + j) of the word's four bytes
+      const uint32_t codes = (15u - 4u * q) | ((14u - 4u * q) << 8) | ((13u - 4u * q) << 16) | ((12u - 4u * q) << 24);
+      const uint32_t k01 = __builtin_amdgcn_perm(ws[q], codes, 0x05010400u);  // (u1, code1, u0, code0)
+      const uint32_t k23 = __builtin_amdgcn_perm(ws[q], codes, 0x07030602u);  // (u3, code3, u2, code2)
+      m = pk_max_u16(m, pk_max_u16(k01, k23));
+    }
+    const uint32_t lo = m & 0xFFFFu, hi = m >> 16;
+    const uint32_t key = lo > hi ? lo : hi;
+    // back to the value's own scale for the comparison with the running best
+    const int v = want_max ? static_cast<int>(key >> 8) - 128 : 127 - static_cast<int>(key >> 8);
+    take(v, static_cast<uint32_t>(i) + 15u - (key & 0xFFu));
   };
   size_t i = static_cast<size_t>(lane) * 16;
   for (; i + 3 * kWave * 16 < whole; i += 4 * kWave * 16) {   // four loads in flight per lane, taken in ascending order
