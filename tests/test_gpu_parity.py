@@ -1855,6 +1855,24 @@ def test_integer_domain_ops_random_configurations(dev):
     assert done["slice"] >= 40 and done["select"] >= 15 and done["expand"] >= 15 and done["arg"] >= 15, done
 
 
+@pytest.mark.parametrize("shape", [(37, 1000), (5, 8240), (3, 4, 16400), (64, 64), (9, 77)])
+def test_q_arg_along_long_and_ragged_rows(dev, shape):
+    """q_argmax / q_argmin along the last dim where the wave-per-row kernel walks several 16-byte pieces per
+    lane, rows that do not start on 16-byte boundaries, tails shorter than a piece, and many ties (values
+    quantized to a few levels): the first index of the extreme, as numpy's."""
+    rng = np.random.default_rng(shape[-1])
+    x = np.round(rng.standard_normal(shape) * 3).astype(np.float32)          # few distinct levels: ties everywhere
+    x[..., -1] = x.max() if shape[-1] % 2 else x.min()                      # an extreme in the ragged tail
+    scheme = QuantScheme(value=QuantValue.Q8S, store=QuantStore.Native)
+    tq = QTensorOps.quantize_dynamic(FloatOps.float_from_data(x, dev), scheme)
+    q_ref, _ = co.quantize_dynamic(x, oscheme(scheme))
+    last = len(shape) - 1
+    for dtype in (ba.I32, ba.I64):
+        assert (IntOps.int_into_data(QTensorOps.q_argmax(tq, last, dtype)) == np.expand_dims(q_ref.argmax(axis=last), last)).all()
+        assert (IntOps.int_into_data(QTensorOps.q_argmin(tq, last, dtype)) == np.expand_dims(q_ref.argmin(axis=last), last)).all()
+    assert (IntOps.int_into_data(QTensorOps.q_argmax(tq, 0)) == np.expand_dims(q_ref.argmax(axis=0), 0)).all()
+
+
 def _int8(dev, floats):
     """The reference tests' QTensor::int8: quantize_dynamic, Q8S per tensor (native store, as the backends
     that run them; crates/burn-backend-tests/tests/tensor/float/quantization/mod.rs:23-50)."""
