@@ -1873,6 +1873,30 @@ def test_q_arg_along_long_and_ragged_rows(dev, shape):
     assert (IntOps.int_into_data(QTensorOps.q_argmax(tq, 0)) == np.expand_dims(q_ref.argmax(axis=0), 0)).all()
 
 
+def test_integer_domain_ops_on_two_level_and_narrow_scale_tensors(dev):
+    """Slices, selects and expands of tensors whose block scales are stored narrow (f16 / ue4m3), alone or
+    under an f32 per-tensor scale: the result dequantizes to the op on the dequantized source bit for bit,
+    and its blob (stored block scales, per-tensor scale) survives q_into_data -> q_from_data."""
+    x = awkward((12, 6, 128), 4242)
+    for scheme in (QuantScheme(value=QuantValue.Q8S).per_block((32,), ScaleDtype.F16).per_tensor(ScaleDtype.F32),
+                   QuantScheme(value=QuantValue.Q4S).per_block((32,), ScaleDtype.UE4M3).per_tensor(ScaleDtype.F32),
+                   QuantScheme(value=QuantValue.Q8S).per_block((32,), ScaleDtype.BF16)):
+        tq = QTensorOps.quantize_dynamic(FloatOps.float_from_data(x, dev), scheme)
+        d = FloatOps.float_into_data(QTensorOps.dequantize(tq))
+        idx = np.int64([11, 0, 3, 3, 7])
+        for got_t, want in ((QTensorOps.q_slice(tq, (slice(2, 10, 3), slice(None, None, -1), slice(32, 128))), d[2:10:3, ::-1, 32:128]),
+                            (QTensorOps.q_select(tq, 0, IntOps.int_from_data(idx, dev)), d[idx]),
+                            (QTensorOps.q_expand(QTensorOps.q_slice(tq, (slice(4, 5),)), (3, 6, 128)), np.broadcast_to(d[4:5], (3, 6, 128)))):
+            assert got_t.scheme == scheme
+            got = FloatOps.float_into_data(QTensorOps.dequantize(got_t))
+            assert got.tobytes() == np.ascontiguousarray(want).tobytes()
+            blob = QTensorOps.q_into_data(got_t)
+            assert blob.bytes.size == TensorData.data_len(got_t.shape, scheme)
+            again = QTensorOps.q_from_data(blob, dev)
+            assert FloatOps.float_into_data(QTensorOps.dequantize(again)).tobytes() == got.tobytes()
+            assert QTensorOps.q_into_data(again).bytes.tobytes() == blob.bytes.tobytes()
+
+
 def _int8(dev, floats):
     """The reference tests' QTensor::int8: quantize_dynamic, Q8S per tensor (native store, as the backends
     that run them; crates/burn-backend-tests/tests/tensor/float/quantization/mod.rs:23-50)."""
