@@ -553,8 +553,23 @@ def run_reference_bench(ba, dev, steps, warmup, cpu):
     def pattern(n):
         return ((np.arange(n) % 1000).astype(np.float32) / np.float32(1000.0) - np.float32(0.5))
 
-    out = {"what": "call + device sync, median of 200, microseconds; the reference's published medians are its CPU backend's "
-                   "on another machine (BASELINE.md)", "scheme": "Q8S per tensor, Native store"}
+    out = {"what": "call + device sync, median of 200, microseconds, timed from Python; `from_c` is the same benchmark timed by "
+                   "the plain-C caller (tests/cpp/c_abi_driver --latency, medians of 400)",
+           "scheme": "Q8S per tensor, Native store",
+           "published_by_the_reference": {
+               "what": "medians of its CPU backends on an Apple M3 Max (crates/burn-flex/BENCHMARKS.md:776-806), microseconds; "
+                       "quantize includes building the tensor from host data, as quantize_with_upload_us does here",
+               "ndarray": {"quantize": {"4K": 10.4, "64K": 145, "1M": 2310}, "dequantize": {"4K": 48.8, "64K": 801, "1M": 13000},
+                           "q_matmul": {"64x64": 137, "256x256": 1930, "512x512": 8070}},
+               "flex": {"quantize": {"4K": 6.93, "64K": 109, "1M": 1750}, "dequantize": {"4K": 0.399, "64K": 3.73, "1M": 54.6},
+                        "q_matmul": {"64x64": 7.10, "256x256": 147, "512x512": 641}}}}
+    driver = os.path.join(ROOT, "tests", "cpp", "c_abi_driver")
+    if os.path.exists(driver):
+        import subprocess
+        r = subprocess.run([driver, "--latency"], capture_output=True, text=True, timeout=300)
+        if r.returncode != 0:
+            raise RuntimeError(f"c_abi_driver --latency failed: {r.stderr[-400:]}")
+        out["from_c"] = json.loads(r.stdout.strip().splitlines()[-1])
     for name, n in (("4K", 64 * 64), ("64K", 256 * 256), ("1M", 1024 * 1024)):
         host = pattern(n)
         x = FloatOps.float_from_data(host, dev)

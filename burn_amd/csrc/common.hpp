@@ -101,6 +101,20 @@ struct bq_device {
   hipEvent_t stage_ev[2] = {nullptr, nullptr};
   bool stage_pending[2] = {false, false};         // a copy out of this half may still be in flight
   int stage_next = 0;
+  // Small uploads and the short wait (set up when the device is opened). A copy of up to kSmallUpload bytes
+  // leaves one of kSmallSlots pinned slots by a copy kernel that writes its sequence number to the slot's
+  // pinned word once it holds the data: the host knows when it may refill a slot by reading memory, with no
+  // event (recording one adds 5 us to a transfer of 3). The last word is written by the kernel bq_device_sync
+  // queues behind everything else.
+  static constexpr size_t kSmallUpload = 64u << 10;
+  static constexpr int kSmallSlots = 4;
+  char* small_stage = nullptr;                    // kSmallSlots * kSmallUpload bytes, pinned
+  uint32_t* host_words = nullptr;                 // kSmallSlots + 1 pinned words the device writes
+  uint32_t small_issued[kSmallSlots] = {};        // sequence number of the last copy queued out of each slot
+  uint32_t small_seq = 0;
+  int small_next = 0;
+  std::mutex sync_mu;                             // orders the wait kernels of concurrent bq_device_sync calls
+  uint32_t sync_seq = 0;
 
   // *actual receives the size of the block handed out (at least `bytes`); pass it to release().
   bq_status alloc(size_t bytes, void** out, size_t* actual);  // stream-ordered reuse is safe: one stream
@@ -112,6 +126,7 @@ struct bq_device {
   bq_status upload(void* dst, const void* src_host, size_t bytes);
   bq_status download(void* dst_host, const void* src, size_t bytes);
   bq_status ensure_stage();
+  bq_status wait_idle();                           // everything queued on the stream has finished
   bq_status trim();
 };
 
@@ -157,6 +172,8 @@ bq_status launch_quantize_rect(const float* x, const size_t* shape, int rank, co
 // Fused quantize kernels with the scheme's scale dtype (quantize.hip). Per tensor: `scale_or_cells`
 // is the scale, or (from_absmax) the absmax cells of pass 1, the derived scale then goes to
 // scale_out. Run blocks: scales_in null = dynamic (scales_out receives them).
+bq_status launch_quantize_per_tensor_small(const float* x, size_t n, float* scale_out, int value, int store, void* values,
+                                           int sdt, hipStream_t stream, bool* done);
 bq_status launch_quantize_per_tensor(const float* x, size_t n, const float* scale_or_cells, bool from_absmax,
                                      float* scale_out, int value, int store, void* values, int scale_dtype,
                                      hipStream_t stream);
@@ -254,6 +271,13 @@ bq_status launch_splitk_reduce(const float* part, size_t mn, unsigned slices, co
 
 // dst[0..n) = value, as a kernel (safe to record into a HIP graph, unlike a memset node).
 bq_status launch_fill_u32(uint32_t* dst, size_t n, uint32_t value, hipStream_t stream);
+// dst[0..bytes) = src[0..bytes) by one workgroup (both 16-byte aligned, bytes <= 64 KiB), then *done = seq
+// at system scope. One side is pinned host memory: when the host sees seq, src has been read (an upload) or
+// dst holds the data (to_host, a download).
+bq_status launch_copy_small(const void* src, void* dst, size_t bytes, bool to_host, uint32_t* done, uint32_t seq,
+                            hipStream_t stream);
+// *word = seq at system scope, behind everything queued on the stream before it.
+bq_status launch_host_word(uint32_t* word, uint32_t seq, hipStream_t stream);
 
 // Host-side guard of a kernel's dynamic LDS request (runtime.cpp). A request beyond what the
 // current device grants is refused here with BQ_ERR_HIP: it must never reach a launch. The first

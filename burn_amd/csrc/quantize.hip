@@ -411,6 +411,60 @@ quantize_tensor_kernel(const float* __restrict__ x, size_t n, const float* __res
   }
 }
 
+// Small tensors: one launch. One workgroup of 1024 threads loads the tensor once (16 floats a lane), takes
+// the maximum through LDS, and quantizes what it holds: the same arithmetic as the two passes, in one
+// dispatch. What a call of this size costs is the launches, not the bytes (a launch and the wait for it
+// take 10.8 us on this part, every further launch 2.3 us, and the second pass cannot start before the first
+// has left the chip): 4096 values 16.2 -> 12.7 us per synchronised call. The limit is where one compute
+// unit's load bandwidth eats the gain: 65 536 values (64 floats a lane) took 16.7 us either way.
+constexpr int kSmallThreads = 1024;
+constexpr size_t kSmallValues = 16384;
+
+template <int VPL, bool FULL>
+__global__ void __launch_bounds__(kSmallThreads)
+quantize_tensor_small_kernel(const float* __restrict__ x, size_t n, float* __restrict__ scale_out,
+                             uint32_t* __restrict__ out, int sdt) {
+  constexpr int U = static_cast<int>(kSmallValues / (kSmallThreads * VPL));
+  constexpr float QMAX = qmax_of(VPL), QMIN = FULL ? -QMAX - 1.0f : -QMAX;
+  __shared__ float part[kSmallThreads / kWave];
+  const size_t words = n / VPL;
+  Vals<VPL> a[U];
+  float m = 0.0f;
+#pragma unroll
+  for (int u = 0; u < U; ++u) {
+    const size_t w = threadIdx.x + static_cast<size_t>(u) * kSmallThreads;
+    if (w < words) {
+      a[u] = load_vals<VPL>(x, w);
+    } else {
+#pragma unroll
+      for (int i = 0; i < VPL; ++i) a[u].v[i] = 0.0f;
+    }
+  }
+#pragma unroll
+  for (int u = 0; u < U; ++u) m = fmaxf(m, absmax_vals<VPL>(a[u]));
+  if (VPL == 4 && threadIdx.x < (n & 3)) m = fmaxf(m, fabsf(x[words * 4 + threadIdx.x]));  // native i8: the last 1..3 values
+  m = group_max<kWave>(m);
+  if ((threadIdx.x & (kWave - 1)) == 0) part[threadIdx.x / kWave] = m;
+  __syncthreads();
+  float amax = part[0];
+#pragma unroll
+  for (int i = 1; i < kSmallThreads / kWave; ++i) amax = fmaxf(amax, part[i]);
+  const float s_stored = scale_round_up(scale_from_absmax(amax, QMAX - QMIN), sdt);
+  if (threadIdx.x == 0) scale_out[0] = s_stored;
+  const float s = valid_scale(s_stored);
+  const bool fast = recip_path_ok(s);
+  const float r = recip_exact(s);
+#pragma unroll
+  for (int u = 0; u < U; ++u) {
+    const size_t w = threadIdx.x + static_cast<size_t>(u) * kSmallThreads;
+    if (w < words) out[w] = fast ? quantize_pack_recip<VPL, true, FULL>(a[u], s, r) : quantize_pack_div<VPL, FULL>(a[u], s);
+  }
+  if (VPL == 4 && threadIdx.x == 0) {
+    int8_t* bytes = reinterpret_cast<int8_t*>(out);
+    for (size_t i = words * 4; i < n; ++i) bytes[i] = static_cast<int8_t>(quantize_div(x[i], s, QMIN, QMAX));
+  }
+}
+
 // 2-bit values against a given scale: 16 values to the word, so a lane that owned a whole word would
 // read 64 bytes at a stride of 64 (the per-tensor kernel above does, at 3.6 TB/s). Here a lane takes
 // one 16-byte piece per load, consecutive lanes consecutive pieces: the four lanes of a quad hold the
@@ -578,6 +632,58 @@ bool fused_block_ok(int block, int value) {
 __global__ void fill_u32_kernel(uint32_t* __restrict__ dst, size_t n, uint32_t value) {
   size_t i = static_cast<size_t>(blockIdx.x) * blockDim.x + threadIdx.x;
   if (i < n) dst[i] = value;
+}
+
+// ---- small host-to-device copies and the word a waiting host reads -----------------------------------------
+// TO_HOST: dst is the pinned memory and the host reads it as soon as it sees seq, so every lane's stores are
+// pushed out to system scope before the barrier.
+template <bool TO_HOST>
+__global__ void __launch_bounds__(1024)
+copy_small_kernel(const vuint4* __restrict__ src, vuint4* __restrict__ dst, uint32_t bytes, uint32_t* __restrict__ done,
+                  uint32_t seq) {
+  const uint32_t n16 = bytes / 16;
+  vuint4 v[4];
+#pragma unroll
+  for (int u = 0; u < 4; ++u) {
+    const uint32_t i = threadIdx.x + u * 1024u;
+    if (i < n16) v[u] = src[i];
+  }
+  uint8_t last = 0;
+  if (threadIdx.x < (bytes & 15u)) last = reinterpret_cast<const uint8_t*>(src)[n16 * 16 + threadIdx.x];
+#pragma unroll
+  for (int u = 0; u < 4; ++u) {
+    const uint32_t i = threadIdx.x + u * 1024u;
+    if (i < n16) dst[i] = v[u];
+  }
+  if (threadIdx.x < (bytes & 15u)) reinterpret_cast<uint8_t*>(dst)[n16 * 16 + threadIdx.x] = last;
+  // a lane's stores were issued with the data its loads brought: behind the barrier no lane reads src any more
+  if (TO_HOST) __threadfence_system();
+  __syncthreads();
+  if (threadIdx.x == 0) __hip_atomic_store(done, seq, TO_HOST ? __ATOMIC_RELEASE : __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+}
+
+__global__ void host_word_kernel(uint32_t* __restrict__ word, uint32_t seq) {
+  if (threadIdx.x == 0) __hip_atomic_store(word, seq, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_SYSTEM);
+}
+
+bq_status launch_copy_small(const void* src, void* dst, size_t bytes, bool to_host, uint32_t* done, uint32_t seq,
+                            hipStream_t st) {
+  if (bytes > 4u * 1024u * 16u || ((reinterpret_cast<uintptr_t>(src) | reinterpret_cast<uintptr_t>(dst)) & 15u))
+    BQ_FAIL(BQ_ERR_SIZE, "small copy of %zu bytes: at most 64 KiB between 16-byte aligned buffers", bytes);
+  if (to_host)
+    hipLaunchKernelGGL(copy_small_kernel<true>, dim3(1), dim3(1024), 0, st, static_cast<const vuint4*>(src),
+                       static_cast<vuint4*>(dst), static_cast<uint32_t>(bytes), done, seq);
+  else
+    hipLaunchKernelGGL(copy_small_kernel<false>, dim3(1), dim3(1024), 0, st, static_cast<const vuint4*>(src),
+                       static_cast<vuint4*>(dst), static_cast<uint32_t>(bytes), done, seq);
+  BQ_HIP(hipGetLastError());
+  return BQ_OK;
+}
+
+bq_status launch_host_word(uint32_t* word, uint32_t seq, hipStream_t st) {
+  hipLaunchKernelGGL(host_word_kernel, dim3(1), dim3(64), 0, st, word, seq);
+  BQ_HIP(hipGetLastError());
+  return BQ_OK;
 }
 
 bq_status launch_fill_u32(uint32_t* dst, size_t n, uint32_t value, hipStream_t st) {
@@ -1228,6 +1334,27 @@ extern "C" bq_status bqk_copy(const void* src, void* dst, size_t bytes, void* st
 namespace bq {
 
 // The handle level's entry into the fused kernels, with the scheme's scale dtype.
+// quantize_dynamic per tensor in one launch, where the tensor is small enough (*done says whether it was):
+// 8-bit values or packed 4-bit ones, a 16-byte aligned input, at most kSmallValues values.
+bq_status launch_quantize_per_tensor_small(const float* x, size_t n, float* scale_out, int value, int store, void* values,
+                                           int sdt, hipStream_t st, bool* done) {
+  *done = false;
+  const int bits = value_bits(value);
+  if (n == 0 || n > kSmallValues || bits == 2 || (bits == 4 && store != BQ_STORE_PACKED_U32) || !aligned16(x) ||
+      (reinterpret_cast<uintptr_t>(values) & 3u))
+    return BQ_OK;
+  BQ_TRY(check_value_store(value, store, n));
+  const bool full = value_full(value);
+  uint32_t* out = static_cast<uint32_t*>(values);
+#define BQ_SMALL(V, F) hipLaunchKernelGGL((quantize_tensor_small_kernel<V, F>), dim3(1), dim3(kSmallThreads), 0, st, x, n, scale_out, out, sdt)
+  if (bits == 8) { if (full) BQ_SMALL(4, true); else BQ_SMALL(4, false); }
+  else { if (full) BQ_SMALL(8, true); else BQ_SMALL(8, false); }
+#undef BQ_SMALL
+  BQ_HIP(hipGetLastError());
+  *done = true;
+  return BQ_OK;
+}
+
 bq_status launch_quantize_per_tensor(const float* x, size_t n, const float* scale_or_cells, bool from_absmax,
                                      float* scale_out, int value, int store, void* values, int sdt, hipStream_t st) {
   return quantize_per_tensor_impl(x, n, scale_or_cells, from_absmax, scale_out, value, store, values, sdt, st);

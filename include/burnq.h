@@ -105,7 +105,10 @@ bq_status bq_device_count(int32_t* count);
  * bq_device_close; handles keep a pointer to theirs. */
 bq_status bq_device_open(int32_t ordinal, bq_device** out);
 bq_status bq_device_close(bq_device* dev);
-/* Backend::sync(device) -- base.rs:154-249: blocks until everything enqueued has finished. */
+/* Backend::sync(device) -- base.rs:154-249: blocks until everything enqueued has finished. (It queues one
+ * small kernel of its own that reports through pinned memory, and reads that memory for a short while before
+ * it blocks in the runtime: 4-5 us sooner than hipStreamSynchronize after short work. Not while a graph is
+ * being captured: an error, as hipStreamSynchronize gives there.) */
 bq_status bq_device_sync(bq_device* dev);
 /* The hipStream_t all work of this context is enqueued on. */
 void* bq_device_stream(bq_device* dev);

@@ -5,6 +5,8 @@
  *
  *   c_abi_driver            needs a GPU: quantize / dequantize / q_matmul / layout cases
  *   c_abi_driver --no-gpu   host-only entry points (sizes, refusals), runs anywhere
+ *   c_abi_driver --latency  needs a GPU: the call latencies of the reference's own quantization benchmark
+ *                           (crates/burn-backend-tests/benches/quantization_ops.rs:26-205), one JSON line
  *
  * Expected values are the literals of burn's tests:
  *   crates/burn-ndarray/src/ops/quantization.rs:164-177            (x -> q, q -> x^)
@@ -13,10 +15,12 @@
  *   crates/burn-store/src/tensor_snapshot.rs:517-541               (packed Q4 data_len)
  *   crates/burn-backend-tests/tests/tensor/float/quantization/ops/matmul.rs:141-168
  */
+#define _POSIX_C_SOURCE 200809L /* clock_gettime under -std=c99 */
 #include <math.h>
 #include <stdio.h>
 #include <stdlib.h>
 #include <string.h>
+#include <time.h>
 
 #include "burnq.h"
 
@@ -179,7 +183,115 @@ static void matmul_case(bq_device* dev) {
   }
 }
 
+/* ---- the reference's benchmark, timed from C ----------------------------------------------------
+ * Per-tensor Q8S, Native store, inputs (i % 1000) / 1000 - 0.5, every call followed by a device sync
+ * (`bench_synced`): `quantize` builds the tensor from host data inside the timed call (make_tensor in
+ * the closure, quantization_ops.rs:63-80), `dequantize` and `q_matmul` work on tensors made before.
+ * Medians of 400 calls after 20 untimed ones, microseconds. */
+static double now_us(void) {
+  struct timespec ts;
+  clock_gettime(CLOCK_MONOTONIC, &ts);
+  return (double)ts.tv_sec * 1e6 + (double)ts.tv_nsec * 1e-3;
+}
+
+static int cmp_double(const void* a, const void* b) {
+  const double x = *(const double*)a, y = *(const double*)b;
+  return (x > y) - (x < y);
+}
+
+enum { LAT_REPS = 400, LAT_WARM = 20 };
+
+typedef struct lat_case {
+  bq_device* dev;
+  const float* host;
+  size_t shape[2];
+  int rank;
+  bq_scheme scheme;
+  bq_tensor *x, *q, *q2;
+} lat_case;
+
+static void lat_sync(lat_case* c) { (void)c; }
+static void lat_upload_quantize(lat_case* c) {
+  bq_tensor *x = NULL, *q = NULL;
+  OK(bq_float_from_data(c->dev, c->host, BQ_F32, c->shape, c->rank, &x));
+  OK(bq_quantize_dynamic(x, &c->scheme, &q));
+  OK(bq_tensor_release(x));
+  OK(bq_tensor_release(q));
+}
+static void lat_quantize(lat_case* c) {
+  bq_tensor* q = NULL;
+  OK(bq_quantize_dynamic(c->x, &c->scheme, &q));
+  OK(bq_tensor_release(q));
+}
+static void lat_dequantize(lat_case* c) {
+  bq_tensor* y = NULL;
+  OK(bq_dequantize(c->q, BQ_F32, &y));
+  OK(bq_tensor_release(y));
+}
+static void lat_matmul(lat_case* c) {
+  bq_tensor* y = NULL;
+  OK(bq_q_matmul(c->q, c->q2, &y));
+  OK(bq_tensor_release(y));
+}
+
+static double median_us(void (*fn)(lat_case*), lat_case* c) {
+  static double t[LAT_REPS];
+  for (int i = 0; i < LAT_WARM; ++i) {
+    fn(c);
+    OK(bq_device_sync(c->dev));
+  }
+  for (int i = 0; i < LAT_REPS; ++i) {
+    const double t0 = now_us();
+    fn(c);
+    OK(bq_device_sync(c->dev));
+    t[i] = now_us() - t0;
+  }
+  qsort(t, LAT_REPS, sizeof t[0], cmp_double);
+  return 0.5 * (t[LAT_REPS / 2 - 1] + t[LAT_REPS / 2]);
+}
+
+static void latency(bq_device* dev) {
+  static const struct { const char* name; size_t rows, cols; } sizes[] = {
+      {"4K", 64, 64}, {"64K", 256, 256}, {"1M", 1024, 1024}, {"q_matmul", 64, 64}, {"q_matmul", 256, 256}, {"q_matmul", 512, 512}};
+  lat_case c;
+  memset(&c, 0, sizeof c);
+  c.dev = dev;
+  c.scheme = scheme_of(BQ_Q8S, BQ_STORE_NATIVE, 0);
+  printf("{\"sync_only_us\": %.2f", median_us(lat_sync, &c));
+  for (size_t s = 0; s < sizeof sizes / sizeof sizes[0]; ++s) {
+    const size_t n = sizes[s].rows * sizes[s].cols;
+    float* host = (float*)malloc(n * sizeof(float));
+    for (size_t i = 0; i < n; ++i) host[i] = (float)(i % 1000) / 1000.0f - 0.5f;
+    c.host = host;
+    const int matmul = sizes[s].name[0] == 'q';
+    c.rank = matmul ? 2 : 1;
+    c.shape[0] = matmul ? sizes[s].rows : n;
+    c.shape[1] = sizes[s].cols;
+    OK(bq_float_from_data(dev, host, BQ_F32, c.shape, c.rank, &c.x));
+    OK(bq_quantize_dynamic(c.x, &c.scheme, &c.q));
+    OK(bq_quantize_dynamic(c.x, &c.scheme, &c.q2));
+    if (matmul) {
+      printf(", \"q_matmul_%zux%zu_us\": %.2f", sizes[s].rows, sizes[s].cols, median_us(lat_matmul, &c));
+    } else {
+      printf(", \"%s\": {\"quantize_with_upload_us\": %.2f, \"quantize_us\": %.2f, \"dequantize_us\": %.2f}", sizes[s].name,
+             median_us(lat_upload_quantize, &c), median_us(lat_quantize, &c), median_us(lat_dequantize, &c));
+    }
+    OK(bq_tensor_release(c.x));
+    OK(bq_tensor_release(c.q));
+    OK(bq_tensor_release(c.q2));
+    free(host);
+  }
+  printf("}\n");
+}
+
 int main(int argc, char** argv) {
+  if (argc > 1 && strcmp(argv[1], "--latency") == 0) {
+    bq_device* dev = NULL;
+    OK(bq_device_open(0, &dev));
+    latency(dev);
+    OK(bq_device_close(dev));
+    return 0;
+  }
   host_only();
   if (argc > 1 && strcmp(argv[1], "--no-gpu") == 0) {
     printf(failures ? "c_abi_driver: %d failure(s)\n" : "c_abi_driver: host-only cases ok\n", failures);

@@ -403,6 +403,25 @@ def test_native_per_tensor_ragged_lengths(dev, n):
     check_quantize_dynamic(dev, x, QuantScheme(store=QuantStore.Native))
 
 
+@pytest.mark.parametrize("n", [8, 4096, 16376, 16384, 16392, 65536])
+def test_small_per_tensor_quantize_one_launch_and_two(dev, n):
+    """Per-tensor quantize_dynamic takes one launch up to 16 384 values and two passes above: the same
+    bits either side of the limit, for every value type and scale dtype the per-tensor kernels take,
+    extreme scales (the division path) and an all-zero tensor (scale 0, quantized against 0.1) included."""
+    x = awkward((n,), n)
+    for scheme in (QuantScheme(store=QuantStore.Native), QuantScheme(), QuantScheme(value=QuantValue.Q4S),
+                   QuantScheme(value=QuantValue.Q8F), QuantScheme(value=QuantValue.Q4F)):
+        check_quantize_dynamic(dev, x, scheme)
+    for sdt in (ScaleDtype.F16, ScaleDtype.BF16, ScaleDtype.UE4M3):
+        check_scale_dtype(dev, x, QuantScheme(scale_dtype=sdt))
+        check_scale_dtype(dev, x, QuantScheme(value=QuantValue.Q4S, scale_dtype=sdt))
+    check_quantize_dynamic(dev, np.zeros(n, np.float32), QuantScheme())
+    check_quantize_dynamic(dev, (x * np.float32(1e-38)).astype(np.float32), QuantScheme(store=QuantStore.Native))
+    check_quantize_dynamic(dev, (x * np.float32(1e36)).astype(np.float32), QuantScheme(value=QuantValue.Q4S))
+    if n % 4 == 0:   # native i8 of a length that is no multiple of 4: the last values go one byte each
+        check_quantize_dynamic(dev, x[: n - 3], QuantScheme(store=QuantStore.Native))
+
+
 def test_empty_tensor(dev):
     x = np.zeros((0, 32), np.float32)
     for scheme in (QuantScheme(store=QuantStore.Native), QuantScheme().per_block((32,))):
