@@ -2027,6 +2027,28 @@ def test_abs_mean_calibration_against_the_oracle(dev, value, shape, block):
 
 # ------------------------------------------------------------------ host threads
 
+def test_small_transfers_through_the_pinned_slots(dev):
+    """Host buffers of at most 64 KiB travel through a few pinned slots that are refilled as soon as a copy
+    kernel has reported: more uploads in a row than there are slots, sizes that are no multiple of 16 bytes,
+    both sides of the 64 KiB limit, each read back, in the order made and in reverse."""
+    rng = np.random.default_rng(77)
+    sizes = [1, 3, 4, 5, 1023, 4096, 16383, 16384, 16385, 1, 16384, 7, 16384 + 4, 2, 16384, 16384, 9]
+    hosts = [rng.standard_normal(n).astype(np.float32) for n in sizes]
+    tensors = [FloatOps.float_from_data(h, dev) for h in hosts]      # 17 uploads, nothing waited for in between
+    for h, t in zip(hosts, tensors):
+        assert FloatOps.float_into_data(t).tobytes() == h.tobytes()
+    for h, t in reversed(list(zip(hosts, tensors))):
+        assert FloatOps.float_into_data(t).tobytes() == h.tobytes()
+    # 2-byte elements: 6 and 65534 bytes
+    for n in (3, 32767, 32768, 32769):
+        bits = rng.integers(0, 1 << 16, n).astype(np.uint16)
+        bits[(bits & 0x7F80) == 0x7F80] = 0x3F80                      # no NaN / Inf patterns
+        t = FloatOps.float_from_data(bits, dev, dtype=ba.BF16)
+        assert FloatOps.float_into_data(t).tobytes() == bits.tobytes()
+    dev.sync()
+    dev.sync()                                                        # a wait with nothing queued returns as well
+
+
 def test_host_threads_share_one_device(dev):
     """crates/burn-backend-tests/tests/tensor/multi_threads.rs: tensors used from several host
     threads at once. Eight threads on one device, each running quantize_dynamic, dequantize and
