@@ -1359,7 +1359,10 @@ static bq_status q_matmul_impl(const bq_tensor* lhs, const bq_tensor* rhs, int32
   }
   // A quantized lhs is dequantized (to f32 when both operands are quantized, as the reference does)
   // and then multiplied like a float one: the weight stays packed and the matrix-core kernels run.
-  const int32_t lhs_dtype = lq ? target : lhs->dtype;
+  // (More than 32 rows always take the tiled kernel, which rounds f32 activations to bf16 on the way in: there
+  // the lhs is dequantized straight to bf16 -- the same bits as f32 and then bf16, one kernel and two passes
+  // over the activations fewer.)
+  const int32_t lhs_dtype = lq ? (target == BQ_F32 && rq && d.m > 32 ? BQ_BF16 : target) : lhs->dtype;
   long run = rq ? run_block(rhs->scheme, rhs->shape, rhs->rank) : -1;
   // (natively stored values of any width are i8s: they multiply as Q8S ones)
   const int rv = rq ? stored_value(rhs->scheme.value, rhs->scheme.store) : BQ_Q8S;
