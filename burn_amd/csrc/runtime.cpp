@@ -428,7 +428,14 @@ extern "C" bq_status bq_device_open(int32_t ordinal, bq_device** out) {
   hipError_t se = hipStreamCreateWithFlags(&dev->stream, hipStreamNonBlocking);
   if (se == hipSuccess) se = hipHostMalloc(reinterpret_cast<void**>(&dev->small_stage), bq_device::kSmallSlots * bq_device::kSmallUpload, hipHostMallocDefault);
   if (se == hipSuccess) se = hipHostMalloc(reinterpret_cast<void**>(&dev->host_words), 64, hipHostMallocDefault);
-  if (se == hipSuccess) std::memset(dev->host_words, 0, 64);
+  if (se == hipSuccess) {
+    // The sequence numbers start 256 short of the 32-bit wrap, so that every process that makes a few
+    // hundred calls goes through it (a server that waits every few microseconds gets there in hours).
+    constexpr uint32_t kFirst = 0xFFFFFF00u;
+    for (int i = 0; i < 16; ++i) dev->host_words[i] = kFirst;
+    for (int i = 0; i < bq_device::kSmallSlots; ++i) dev->small_issued[i] = kFirst;
+    dev->small_seq = dev->sync_seq = kFirst;
+  }
   // the ticket counters of the single-launch split-K sum: zero from here on, every launch leaves them so
   if (se == hipSuccess) se = hipMalloc(reinterpret_cast<void**>(&dev->tickets), kTicketBytes);
   if (se == hipSuccess) se = hipMemset(dev->tickets, 0, kTicketBytes);
