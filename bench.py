@@ -648,6 +648,19 @@ def run_next(ba, dev, steps, warmup, cpu):
                         "max_normalised_error": rel}
     out["q4s_small_batch"] = {"workload": "x[M,4096] f32 x Q4S block-32 PackedU32 [4096,14336] -> f32 (C4's shape, half the weight bytes)",
                               "parity": "vs float64 on every 37th column, rel 1e-2 and burn's elementwise rule", **q4}
+    # batches between the decode kernels (M <= 32) and prefill: the tiled kernel on row tiles it does not fill
+    mid = {}
+    for m in (64, 128, 512):
+        xh = ba.f32_from_bf16_bits(ba.bf16_bits_from_f32(rng.standard_normal((m, k), dtype=np.float32))).reshape(m, k)
+        x = FloatOps.float_from_data(ba.bf16_bits_from_f32(xh), dev, ba.BF16)
+        got = FloatOps.float_into_data(QTensorOps.q_matmul(x, ws[5], out_dtype=ba.F32))[:, cols]
+        rel = matmul_gate(f"Q4S M={m}", got, xh.astype(np.float64) @ wd, max_outside=8)
+        t_mm = graph_ms(dev, lambda: [QTensorOps.q_matmul(x, wq, out_dtype=ba.F32) for wq in ws], 16, steps, warmup)
+        mid[f"M={m}"] = {"ms": t_mm, "TFLOP/s": 2.0 * m * k * n / t_mm / 1e9, "frac_mfma": 2.0 * m * k * n / t_mm / 1e9 / BF16_PEAK_TFLOPS,
+                         "weight_GB/s": wb / t_mm / 1e6, "max_normalised_error": rel}
+    out["q4s_mid_batch"] = {"workload": "x[M,4096] bf16 x Q4S block-32 PackedU32 [4096,14336] -> f32, 64 to 512 rows (C5's operand types)",
+                            "parity": "vs float64 on every 37th column, rel 1e-2; at most 8 outputs outside burn's elementwise rule "
+                                      "(the tiled kernel rounds s * q to bf16)", **mid}
     del ws, w0, blob, values, scales
     dev.trim()
 
