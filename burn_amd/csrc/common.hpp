@@ -291,10 +291,21 @@ bq_status static_scratch_ptr(void** out, unsigned** tickets_out = nullptr);
 // bqk_q_linear plus the ticket counters that let the split-K kernels finish their own sum in one
 // launch (qmatmul.hip, splitk_tail.hpp): `tickets` is kTicketBytes of device memory, zero between
 // launches; calls sharing it must not overlap on the device.
+// QuantPropagation::Propagate without a float product in memory: where a product ends in the reduction of its
+// K slices, that kernel can quantize what it sums -- blocks of 32 or 64 output columns, the scale of each
+// from its own absmax -- into `values` / `scales` of a quantized tensor. `done` says whether it did (the
+// float output is then not written).
+struct RequantOut {
+  int value = 0, store = 0, block = 0, sdt = 0;
+  bool from_bf16 = false;  // the product is a bf16 tensor: its values are rounded to bf16 before they are quantized
+  void* values = nullptr;
+  float* scales = nullptr;
+  bool done = false;
+};
 bq_status q_linear_with_tickets(const void* x, int32_t x_dtype, size_t m, size_t k, size_t n, const void* w_values,
                                 const float* w_scales, int32_t block, int32_t value, int32_t store, const float* bias,
                                 int32_t out_dtype, void* out, void* workspace, size_t workspace_bytes, unsigned* tickets,
-                                void* stream);
+                                void* stream, RequantOut* requant = nullptr);
 
 // Counts, over n floats, NaNs into counts[0] and infinities into counts[1] (device u32 cells that
 // the kernel adds to; quantize.hip). Used by the validate mode.

@@ -319,10 +319,9 @@ qgemv1_kernel(const void* __restrict__ x, const uint32_t* __restrict__ w,
 // lanes" each add every SL-th slice in ascending order, then lane 0 adds the SL subtotals in
 // ascending order: a fixed summation tree, so results are reproducible run to run. SL is the
 // largest of 16, 8, 4 that does not exceed the slice count (no idle slice lanes).
-template <bool BF16, int SL>
-__global__ void __launch_bounds__(256)
-qgemv_reduce_kernel(const float* __restrict__ part, size_t mn, unsigned slices, const float* __restrict__ bias,
-                    size_t n, void* __restrict__ out) {
+template <int SL>
+__device__ __forceinline__ bool reduce_slices(const float* __restrict__ part, size_t mn, unsigned slices,
+                                              const float* __restrict__ bias, size_t n, size_t& i_out, vfloat4& v_out) {
   constexpr int COLS = 256 / SL;
   __shared__ vfloat4 sub[SL][COLS];
   const int c = threadIdx.x % COLS, sl = threadIdx.x / COLS;
@@ -344,7 +343,8 @@ qgemv_reduce_kernel(const float* __restrict__ part, size_t mn, unsigned slices, 
   }
   sub[sl][c] = v;
   __syncthreads();
-  if (sl == 0 && i < mn) {
+  const bool mine = sl == 0 && i < mn;
+  if (mine) {
 #pragma unroll
     for (int t = 1; t < SL; ++t) v += sub[t][c];
     if (bias != nullptr) {  // the linear layer's bias, added last: (sum of products) + bias[column]
@@ -358,6 +358,20 @@ qgemv_reduce_kernel(const float* __restrict__ part, size_t mn, unsigned slices, 
         v.w += bias[(i + 3) % n];
       }
     }
+  }
+  i_out = i;
+  v_out = v;
+  return mine;  // this thread holds outputs i .. i + 3
+}
+
+template <bool BF16, int SL>
+__global__ void __launch_bounds__(256)
+qgemv_reduce_kernel(const float* __restrict__ part, size_t mn, unsigned slices, const float* __restrict__ bias,
+                    size_t n, void* __restrict__ out) {
+  size_t i;
+  vfloat4 v;
+  if (reduce_slices<SL>(part, mn, slices, bias, n, i, v)) {
+    const bool vec = (mn & 3) == 0;
     const float r[4] = {v.x, v.y, v.z, v.w};
     if (vec && !BF16) {
       *reinterpret_cast<vfloat4*>(static_cast<float*>(out) + i) = v;
@@ -370,6 +384,46 @@ qgemv_reduce_kernel(const float* __restrict__ part, size_t mn, unsigned slices, 
       }
     }
   }
+}
+
+// The same sum, quantized where it is formed (QuantPropagation::Propagate, crates/burn-ndarray/src/ops/
+// qtensor.rs:262-265, for a block scheme). A block of 4 * LANES consecutive outputs -- 32 or 64 columns of one
+// row, n being a multiple of it -- lies in LANES consecutive lanes: absmax across them by DPP, the scale
+// (2 * absmax) / (b - a) rounded up to the scale dtype, each value divided by it, rounded half away from
+// zero and clamped: the arithmetic of quantize_dynamic on the float product, which is never written.
+// VPL = 4: a lane's four values are one word (or four native bytes). VPL = 8: a word is two lanes' values.
+template <int SL, int VPL, int LANES>
+__global__ void __launch_bounds__(256)
+qgemv_reduce_quant_kernel(const float* __restrict__ part, size_t mn, unsigned slices, const float* __restrict__ bias,
+                          size_t n, float qmin, float qmax, int sdt, int from_bf16, uint32_t* __restrict__ values,
+                          float* __restrict__ scales) {
+  size_t i;
+  vfloat4 v;
+  const bool mine = reduce_slices<SL>(part, mn, slices, bias, n, i, v);
+  // (mn is a multiple of the block: the lanes of a block hold outputs together or not at all; the
+  // cross-lane steps below run in every lane)
+  float r[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+  for (int e = 0; e < 4; ++e) {
+    if (!mine) r[e] = 0.0f;
+    if (from_bf16) r[e] = bf16_to_f32(f32_to_bf16(r[e]));
+  }
+  const float m = group_max<LANES>(fmaxf(fmaxf(fabsf(r[0]), fabsf(r[1])), fmaxf(fabsf(r[2]), fabsf(r[3]))));
+  const float s_stored = scale_round_up(scale_from_absmax(m, qmax - qmin), sdt);
+  const float s = valid_scale(s_stored);
+  int q[4];
+#pragma unroll
+  for (int e = 0; e < 4; ++e) q[e] = quantize_div(r[e], s, qmin, qmax);
+  const int c = threadIdx.x % (256 / SL);
+  if (VPL == 4) {
+    if (mine) values[i / 4] = pack_fields<4>(q);
+  } else {
+    const uint32_t half = static_cast<uint32_t>(q[0] & 15) | static_cast<uint32_t>(q[1] & 15) << 4 |
+                          static_cast<uint32_t>(q[2] & 15) << 8 | static_cast<uint32_t>(q[3] & 15) << 12;
+    const uint32_t next = dpp_lane<0xB1>(half);  // quad_perm [1,0,3,2]: the odd neighbour's half for an even lane
+    if (mine && (c & 1) == 0) values[i / 8] = half | next << 16;
+  }
+  if (mine && (c & (LANES - 1)) == 0) scales[i / (4 * LANES)] = s_stored;
 }
 
 struct GemvPlan {
@@ -694,11 +748,35 @@ extern "C" size_t bqk_q_matmul_workspace(size_t m, size_t k, size_t n, int32_t l
   return std::max(bytes, qgemm_workspace(lhs_dtype, m, k, n));
 }
 
+static bool requant_fits(const RequantOut* rq, size_t mn, size_t n) {
+  if (rq == nullptr || rq->values == nullptr || rq->scales == nullptr) return false;
+  const int bits = value_bits(rq->value);
+  if (!(rq->block == 32 || rq->block == 64) || n % static_cast<size_t>(rq->block) || mn % static_cast<size_t>(rq->block)) return false;
+  if (bits == 8) return rq->store == BQ_STORE_NATIVE || rq->store == BQ_STORE_PACKED_U32;
+  return bits == 4 && rq->store == BQ_STORE_PACKED_U32;
+}
+
 static bq_status launch_gemv_reduce(const float* part, size_t mn, unsigned slices, const float* bias, size_t n,
-                                    int32_t out_dtype, void* out, hipStream_t st) {
+                                    int32_t out_dtype, void* out, hipStream_t st, RequantOut* rq = nullptr) {
   const size_t cols4 = (mn + 3) / 4;
   const int sl = slices >= 16 ? 16 : (slices >= 8 ? 8 : 4);
   dim3 grid(static_cast<unsigned>((cols4 + 256 / sl - 1) / (256 / sl))), tb(256);
+  if (requant_fits(rq, mn, n)) {
+    const float qmax = static_cast<float>(value_qmax(rq->value)), qmin = static_cast<float>(value_qmin(rq->value));
+    const int vpl = value_bits(rq->value) == 8 ? 4 : 8, lanes = rq->block / 4;
+#define BQ_RQ(S, V, L)                                                                                              \
+  hipLaunchKernelGGL((qgemv_reduce_quant_kernel<S, V, L>), grid, tb, 0, st, part, mn, slices, bias, n, qmin, qmax, \
+                     rq->sdt, rq->from_bf16 ? 1 : 0, static_cast<uint32_t*>(rq->values), rq->scales)
+#define BQ_RQ_S(V, L) \
+  if (sl == 16) BQ_RQ(16, V, L); else if (sl == 8) BQ_RQ(8, V, L); else BQ_RQ(4, V, L)
+    if (vpl == 4) { if (lanes == 8) { BQ_RQ_S(4, 8); } else { BQ_RQ_S(4, 16); } }
+    else { if (lanes == 8) { BQ_RQ_S(8, 8); } else { BQ_RQ_S(8, 16); } }
+#undef BQ_RQ_S
+#undef BQ_RQ
+    BQ_HIP(hipGetLastError());
+    rq->done = true;
+    return BQ_OK;
+  }
 #define BQ_REDUCE(B, S) hipLaunchKernelGGL((qgemv_reduce_kernel<B, S>), grid, tb, 0, st, part, mn, slices, bias, n, out)
   if (out_dtype == BQ_BF16) {
     if (sl == 16) BQ_REDUCE(true, 16); else if (sl == 8) BQ_REDUCE(true, 8); else BQ_REDUCE(true, 4);
@@ -733,7 +811,8 @@ static bq_status q_matmul_core(const void* lhs, int32_t lhs_dtype, size_t m, siz
                                const void* w_values, const float* w_scales, int32_t block,
                                int32_t value, int32_t store, const float* bias, int32_t out_dtype, void* out,
                                void* workspace, size_t workspace_bytes, void* stream, size_t* need_out = nullptr,
-                               unsigned* tickets = nullptr) {
+                               unsigned* tickets = nullptr, RequantOut* requant = nullptr) {
+  if (requant != nullptr) tickets = nullptr;  // (the quantizing sum is the reduction kernel's: two launches)
   // tickets: kTicketBytes of device memory, zero between launches (splitk_tail.hpp), or null. With
   // them the decode kernel finishes its own split-K sum for one or two rows: one launch instead of two.
   // need_out: dry run. The arguments are validated and the kernel is chosen as usual, but nothing is
@@ -792,7 +871,7 @@ static bq_status q_matmul_core(const void* lhs, int32_t lhs_dtype, size_t m, siz
     // the reduction kernel reads with the whole chip while a last workgroup per tile would read them
     // alone -- measured on the 4096 x 14336 weight, M = 4 / 16: 20.1 / 25.3 us against 19.8 / 22.5 us)
     BQ_TRY(launch_qsplit(lhs, lhs_dtype, w, w_scales, m, k, n, value, block, part, &slices, st));
-    return launch_gemv_reduce(part, m * n, slices, bias, n, out_dtype, out, st);
+    return launch_gemv_reduce(part, m * n, slices, bias, n, out_dtype, out, st, requant);
   }
 
   if (gemv1_ok(m, n, lhs_dtype, block, value) && (reinterpret_cast<uintptr_t>(w_values) & 15u) == 0 &&
@@ -856,7 +935,7 @@ static bq_status q_matmul_core(const void* lhs, int32_t lhs_dtype, size_t m, siz
 #undef BQ_GEMV1B
     BQ_HIP(hipGetLastError());
     if (tk != nullptr) return BQ_OK;
-    return launch_gemv_reduce(part, m * n, p.slices, bias, n, out_dtype, out, st);
+    return launch_gemv_reduce(part, m * n, p.slices, bias, n, out_dtype, out, st, requant);
   }
 
   // f32 activations: the FP32-matrix kernel pays off from M = 7 (measured: 38-41 us flat against
@@ -872,7 +951,7 @@ static bq_status q_matmul_core(const void* lhs, int32_t lhs_dtype, size_t m, siz
     float* part = static_cast<float*>(workspace);
     unsigned slices = 0;
     BQ_TRY(launch_qskinny(lhs, lhs_dtype, w, w_scales, m, k, n, value, bwl2, spr, per_tensor, part, &slices, st));
-    return launch_gemv_reduce(part, m * n, slices, bias, n, out_dtype, out, st);
+    return launch_gemv_reduce(part, m * n, slices, bias, n, out_dtype, out, st, requant);
   }
 
   if (use_gemv(m, lhs_dtype)) {
@@ -914,7 +993,7 @@ static bq_status q_matmul_core(const void* lhs, int32_t lhs_dtype, size_t m, siz
 #undef BQ_GEMV_M
 #undef BQ_GEMV
     BQ_HIP(hipGetLastError());
-    return launch_gemv_reduce(part, m * n, p.slices, bias, n, out_dtype, out, st);
+    return launch_gemv_reduce(part, m * n, p.slices, bias, n, out_dtype, out, st, requant);
   }
 
   if (!qgemm_ok(lhs_dtype, k, n, value, spr))
@@ -924,7 +1003,7 @@ static bq_status q_matmul_core(const void* lhs, int32_t lhs_dtype, size_t m, siz
   float* part = nullptr;
   BQ_TRY(launch_qgemm(lhs, lhs_dtype, w, w_scales, m, k, n, value, bwl2, spr, per_tensor, bias, out_dtype, out,
                       workspace, workspace_bytes, &slices, &part, st));
-  if (slices > 1) return launch_gemv_reduce(part, m * n, slices, bias, n, out_dtype, out, st);
+  if (slices > 1) return launch_gemv_reduce(part, m * n, slices, bias, n, out_dtype, out, st, requant);
   return BQ_OK;
 }
 
@@ -952,11 +1031,11 @@ namespace bq {
 bq_status q_linear_with_tickets(const void* x, int32_t x_dtype, size_t m, size_t k, size_t n, const void* w_values,
                                 const float* w_scales, int32_t block, int32_t value, int32_t store, const float* bias,
                                 int32_t out_dtype, void* out, void* workspace, size_t workspace_bytes, unsigned* tickets,
-                                void* stream) {
+                                void* stream, RequantOut* requant) {
   if (bias != nullptr && (reinterpret_cast<uintptr_t>(bias) & 15u))
     BQ_FAIL(BQ_ERR_SHAPE, "q_linear bias must be 16-byte aligned");
   return q_matmul_core(x, x_dtype, m, k, n, w_values, w_scales, block, value, store, bias, out_dtype, out,
-                       workspace, workspace_bytes, stream, nullptr, tickets);
+                       workspace, workspace_bytes, stream, nullptr, tickets, requant);
 }
 }  // namespace bq
 

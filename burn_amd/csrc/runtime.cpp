@@ -1314,8 +1314,12 @@ extern "C" bq_status bq_float_matmul(const bq_tensor* lhs, const bq_tensor* rhs,
 }
 
 // `bias` (device f32, N entries, or null) is a linear layer's: added to every row of the product.
+// quantized_out (optional): the caller wants the product quantized again with *requant_scheme (Propagate). Where
+// the product ends in a reduction of K slices that can quantize what it sums, *quantized_out receives that
+// tensor and *out stays null; otherwise *quantized_out stays null and *out is the float product as usual.
 static bq_status q_matmul_impl(const bq_tensor* lhs, const bq_tensor* rhs, int32_t out_dtype_req,
-                               const float* bias, bq_tensor** out) {
+                               const float* bias, bq_tensor** out, bq_tensor** quantized_out = nullptr,
+                               const bq_scheme* requant_scheme = nullptr) {
   BQ_NOTNULL(lhs);
   BQ_NOTNULL(rhs);
   BQ_NOTNULL(out);
@@ -1409,6 +1413,25 @@ static bq_status q_matmul_impl(const bq_tensor* lhs, const bq_tensor* rhs, int32
       if (lf) bq_tensor_release(lf);
       return rc;
     }
+    // Propagate with a scheme of 32 or 64 columns per scale along the last dim (one level): the reduction of the
+    // K slices, where the product has one, writes the quantized tensor
+    RequantOut requant;
+    bq_tensor* qt = nullptr;
+    // (not in validate mode: quantize_dynamic then inspects the float product first)
+    if (quantized_out != nullptr && requant_scheme != nullptr && d.batches == 1 && !dev->validate.load() &&
+        requant_scheme->level == BQ_LEVEL_BLOCK &&
+        !requant_scheme->tensor_scale && fused_value(requant_scheme->value, requant_scheme->store)) {
+      const long out_run = run_block(*requant_scheme, d.out_shape, d.rank);
+      if ((out_run == 32 || out_run == 64) && new_quantized(dev, *requant_scheme, d.out_shape, d.rank, &qt) == BQ_OK) {
+        requant.value = requant_scheme->value;
+        requant.store = requant_scheme->store;
+        requant.block = static_cast<int>(out_run);
+        requant.sdt = requant_scheme->scale_dtype;
+        requant.from_bf16 = out_dtype == BQ_BF16;
+        requant.values = qt->data;
+        requant.scales = qt->scales();
+      }
+    }
     const size_t ws = bqk_q_matmul_workspace(d.m, d.k, d.n, lhs_dtype, rv);
     std::unique_lock<std::mutex> lock(dev->mu, std::defer_lock);
     if (ws) {
@@ -1428,14 +1451,22 @@ static bq_status q_matmul_impl(const bq_tensor* lhs, const bq_tensor* rhs, int32
                                  rhs->scales() + rb * scales_per_batch, static_cast<int32_t>(run), rv,
                                  rhs->scheme.store, bias, out_dtype,
                                  static_cast<char*>(o->data) + b * d.m * d.n * dtype_size(out_dtype), dev->workspace,
-                                 dev->workspace_bytes, lock.owns_lock() ? dev->tickets : nullptr, st);
+                                 dev->workspace_bytes, lock.owns_lock() ? dev->tickets : nullptr, st,
+                                 qt != nullptr ? &requant : nullptr);
     }
     if (lock.owns_lock()) lock.unlock();  // (releasing a tensor takes the same mutex)
     if (lf) bq_tensor_release(lf);         // (stream-ordered: the kernels above were enqueued first)
     if (rc != BQ_OK) {
       bq_tensor_release(o);
+      if (qt) bq_tensor_release(qt);
       return rc;
     }
+    if (qt != nullptr && requant.done) {  // the float product was never written
+      bq_tensor_release(o);
+      *quantized_out = qt;
+      return BQ_OK;
+    }
+    if (qt) bq_tensor_release(qt);
     *out = o;
     return BQ_OK;
   }
@@ -1499,7 +1530,12 @@ extern "C" bq_status bq_q_matmul_propagate(const bq_tensor* lhs, const bq_tensor
   // The product has the float operand's dtype (qtensor.rs:234-239). A bf16 product is what gets
   // quantized: its values, widened exactly to the f32 the quantize kernels read.
   bq_tensor* f = nullptr;
-  BQ_TRY(q_matmul_impl(lhs, rhs, target, nullptr, &f));
+  bq_tensor* quantized = nullptr;
+  BQ_TRY(q_matmul_impl(lhs, rhs, target, nullptr, &f, &quantized, &scheme));
+  if (quantized != nullptr) {  // quantized where the K slices were summed
+    *out = quantized;
+    return BQ_OK;
+  }
   bq_status rc = BQ_OK;
   if (target == BQ_BF16) {
     bq_tensor* wide = nullptr;

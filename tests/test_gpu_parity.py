@@ -2580,6 +2580,41 @@ def test_q_matmul_propagate_requantizes(dev, value, block):
     assert out_b.is_quantized and (q == q_ref).all() and s.tobytes() == s_ref.tobytes()
 
 
+@pytest.mark.parametrize("m", [1, 2, 4, 16, 32, 64, 300, 2048])
+def test_q_matmul_propagate_quantized_in_the_reduction(dev, m):
+    """Propagate with 32 or 64 columns per scale: where the product ends in the sum of its K slices (every batch
+    up to 32 rows, larger ones while the tiled kernel splits K) that kernel writes the quantized tensor and no
+    float product exists; elsewhere two steps. Either way: quantize_dynamic of q_matmul's result, byte for byte,
+    and the CPU oracle's quantization of that product."""
+    rng = np.random.default_rng(100 + m)
+    k, n = 512, 1024
+    w = (rng.standard_normal((k, n)) * 0.05).astype(np.float32)
+    x = rng.standard_normal((m, k)).astype(np.float32)
+    x[rng.random(x.shape) < 0.01] *= 30
+    cases = [QuantScheme().per_block((32,)), QuantScheme().per_block((64,)), QuantScheme(value=QuantValue.Q4S).per_block((32,)),
+             QuantScheme(value=QuantValue.Q4S).per_block((64,)), QuantScheme(store=QuantStore.Native).per_block((32,)),
+             QuantScheme(value=QuantValue.Q8F).per_block((32,)), QuantScheme().per_block((32,), ScaleDtype.F16),
+             QuantScheme().per_block((128,)), QuantScheme()]
+    for scheme in cases:
+        tq = QTensorOps.quantize_dynamic(FloatOps.float_from_data(w, dev), scheme)
+        for tx in (FloatOps.float_from_data(x, dev), FloatOps.float_from_data(ba.bf16_bits_from_f32(x), dev, ba.BF16)):
+            out = QTensorOps.q_matmul_propagate(tx, tq)
+            assert out.is_quantized and out.shape == (m, n)
+            prod_t = QTensorOps.q_matmul(tx, tq)
+            prod = FloatOps.float_into_data(prod_t)
+            if tx.dtype == ba.BF16:
+                prod = ba.f32_from_bf16_bits(prod).reshape(m, n)
+                prod_t = FloatOps.float_from_data(prod, dev)
+            two_steps = QTensorOps.quantize_dynamic(prod_t, scheme)
+            blob = QTensorOps.q_into_data(out)
+            assert blob.bytes.tobytes() == QTensorOps.q_into_data(two_steps).bytes.tobytes(), (scheme, tx.dtype)
+            if scheme.scale_dtype == ScaleDtype.F32:
+                q_ref, s_ref = co.quantize_dynamic(prod, oscheme(scheme))
+                assert blob.bytes.tobytes() == co.encode(q_ref, oscheme(scheme), s_ref).tobytes(), (scheme, tx.dtype)
+    # with a bias the Linear layer adds: not part of Propagate, the plain product is unchanged by all this
+    assert FloatOps.float_into_data(QTensorOps.q_matmul(FloatOps.float_from_data(x, dev), tq)).shape == (m, n)
+
+
 def test_q_matmul_empty_k_is_zero(dev):
     """[M,0] x [0,N]: an empty sum, written as zeros over whatever the output held."""
     from burn_amd import _lib
