@@ -627,6 +627,22 @@ def run_next(ba, dev, steps, warmup, cpu):
         lin[f"M={m}"] = {"ms": t_lin, "ms_without_bias": t_mm, "GB/s": (k * n + 4 * k * n // 32) / t_lin / 1e6}
     out["linear"] = {"workload": "x[M,4096] f32 x Q8S block-32 [4096,14336] + bias[14336] -> f32 (C4's weight)",
                      "parity": "vs float64 on every 37th column, rel 1e-2 and burn's elementwise rule", **lin}
+    # ---- QuantPropagation::Propagate: the product comes back quantized with the weight's scheme -----
+    osch = co.Scheme.make(co.Q8S, [32], co.STORE_PACKED_U32)
+    scheme = ws[0].scheme
+    prop = {}
+    for m in (4, 16):
+        x = FloatOps.float_from_data(rng.standard_normal((m, k), dtype=np.float32), dev)
+        prod = FloatOps.float_into_data(QTensorOps.q_matmul(x, ws[2]))
+        q_ref, s_ref = co.quantize_dynamic(prod, osch)
+        if QTensorOps.q_into_data(QTensorOps.q_matmul_propagate(x, ws[2])).bytes.tobytes() != co.encode(q_ref, osch, s_ref).tobytes():
+            raise ParityError(f"Propagate M={m}: differs from the CPU oracle's quantization of the product")
+        t_p = graph_ms(dev, lambda: [QTensorOps.q_matmul_propagate(x, wq) for wq in ws], 16, steps, warmup)
+        t_2 = graph_ms(dev, lambda: [QTensorOps.quantize_dynamic(QTensorOps.q_matmul(x, wq), scheme) for wq in ws], 16, steps, warmup)
+        prop[f"M={m}"] = {"ms": t_p, "ms_product_then_quantize_dynamic": t_2}
+    out["propagate"] = {"workload": "x[M,4096] f32 x Q8S block-32 [4096,14336] -> Q8S block-32 [M,14336] (C4's weight; the K-slice "
+                                    "reduction quantizes what it sums)",
+                        "parity": "blob bit-exact vs the CPU oracle's quantize_dynamic of the device's float product", **prop}
     del ws, w0, blob, values, scales
     dev.trim()
 
