@@ -419,6 +419,7 @@ def run_c4(ba, dev, steps, warmup, cpu):
     return out
 
 
+NEXT_PART = "all"  # --next-part: "matmul" (Linear, Propagate, Q4S batches, ternary, burnpack) or "tensor" (the rest) alone
 C5_N = 14336  # weight columns of C5; --c5-n runs the same product at another width (tile-count studies)
 
 
@@ -606,258 +607,261 @@ def run_next(ba, dev, steps, warmup, cpu):
     out = {"timing": "HIP graphs over distinct tensors; ms per call"}
     rng = np.random.default_rng(0xF0)
 
-    # ---- quantized Linear: the bias rides in the product's epilogue ------------------------------
-    k, n = 4096, 14336
-    w0 = quantized_weight(ba, dev, 0xC4, (k, n), QuantValue.Q8S)
-    blob = QTensorOps.q_into_data(w0)
-    ws = [w0] + [QTensorOps.q_from_data(blob, dev) for _ in range(15)]
-    values, scales = blob.split()
-    bias_h = rng.standard_normal(n, dtype=np.float32)
-    bias = FloatOps.float_from_data(bias_h, dev)
-    cols = np.arange(0, n, 37)
-    wd = unpack_columns(values, scales, k, n, cols, q4=False)
-    lin = {}
-    for m in (1, 16):
-        xh = rng.standard_normal((m, k), dtype=np.float32)
-        x = FloatOps.float_from_data(xh, dev)
-        got = FloatOps.float_into_data(ModuleOps.linear(x, ws[3], bias))[:, cols]
-        matmul_gate(f"linear M={m}", got, xh.astype(np.float64) @ wd + bias_h[cols].astype(np.float64))
-        t_lin = graph_ms(dev, lambda: [ModuleOps.linear(x, wq, bias) for wq in ws], 16, steps, warmup)
-        t_mm = graph_ms(dev, lambda: [QTensorOps.q_matmul(x, wq) for wq in ws], 16, steps, warmup)
-        lin[f"M={m}"] = {"ms": t_lin, "ms_without_bias": t_mm, "GB/s": (k * n + 4 * k * n // 32) / t_lin / 1e6}
-    out["linear"] = {"workload": "x[M,4096] f32 x Q8S block-32 [4096,14336] + bias[14336] -> f32 (C4's weight)",
-                     "parity": "vs float64 on every 37th column, rel 1e-2 and burn's elementwise rule", **lin}
-    # ---- QuantPropagation::Propagate: the product comes back quantized with the weight's scheme -----
-    osch = co.Scheme.make(co.Q8S, [32], co.STORE_PACKED_U32)
-    scheme = ws[0].scheme
-    prop = {}
-    for m in (4, 16):
-        x = FloatOps.float_from_data(rng.standard_normal((m, k), dtype=np.float32), dev)
-        prod = FloatOps.float_into_data(QTensorOps.q_matmul(x, ws[2]))
-        q_ref, s_ref = co.quantize_dynamic(prod, osch)
-        if QTensorOps.q_into_data(QTensorOps.q_matmul_propagate(x, ws[2])).bytes.tobytes() != co.encode(q_ref, osch, s_ref).tobytes():
-            raise ParityError(f"Propagate M={m}: differs from the CPU oracle's quantization of the product")
-        t_p = graph_ms(dev, lambda: [QTensorOps.q_matmul_propagate(x, wq) for wq in ws], 16, steps, warmup)
-        t_2 = graph_ms(dev, lambda: [QTensorOps.quantize_dynamic(QTensorOps.q_matmul(x, wq), scheme) for wq in ws], 16, steps, warmup)
-        prop[f"M={m}"] = {"ms": t_p, "ms_product_then_quantize_dynamic": t_2}
-    out["propagate"] = {"workload": "x[M,4096] f32 x Q8S block-32 [4096,14336] -> Q8S block-32 [M,14336] (C4's weight; the K-slice "
-                                    "reduction quantizes what it sums)",
-                        "parity": "blob bit-exact vs the CPU oracle's quantize_dynamic of the device's float product", **prop}
-    del ws, w0, blob, values, scales
-    dev.trim()
-
-    # ---- the same products over a 4-bit weight ------------------------------------------------------
-    w0 = quantized_weight(ba, dev, 0xC4, (k, n), QuantValue.Q4S)
-    blob = QTensorOps.q_into_data(w0)
-    ws = [w0] + [QTensorOps.q_from_data(blob, dev) for _ in range(15)]
-    values, scales = blob.split()
-    wd = unpack_columns(values, scales, k, n, cols, q4=True)
-    q4 = {}
-    for m in (1, 4, 16):
-        xh = rng.standard_normal((m, k), dtype=np.float32)
-        x = FloatOps.float_from_data(xh, dev)
-        got = FloatOps.float_into_data(QTensorOps.q_matmul(x, ws[5]))[:, cols]
-        rel = matmul_gate(f"Q4S M={m}", got, xh.astype(np.float64) @ wd)
-        t_mm = graph_ms(dev, lambda: [QTensorOps.q_matmul(x, wq) for wq in ws], 16, steps, warmup)
-        wb = k * n // 2 + 4 * k * n // 32
-        q4[f"M={m}"] = {"ms": t_mm, "weight_GB/s": wb / t_mm / 1e6, "frac_hbm": wb / t_mm / 1e6 / HBM_PEAK_GBS,
-                        "max_normalised_error": rel}
-    out["q4s_small_batch"] = {"workload": "x[M,4096] f32 x Q4S block-32 PackedU32 [4096,14336] -> f32 (C4's shape, half the weight bytes)",
-                              "parity": "vs float64 on every 37th column, rel 1e-2 and burn's elementwise rule", **q4}
-    # batches between the decode kernels (M <= 32) and prefill: the tiled kernel on row tiles it does not fill
-    mid = {}
-    for m in (64, 128, 512):
-        xh = ba.f32_from_bf16_bits(ba.bf16_bits_from_f32(rng.standard_normal((m, k), dtype=np.float32))).reshape(m, k)
-        x = FloatOps.float_from_data(ba.bf16_bits_from_f32(xh), dev, ba.BF16)
-        got = FloatOps.float_into_data(QTensorOps.q_matmul(x, ws[5], out_dtype=ba.F32))[:, cols]
-        rel = matmul_gate(f"Q4S M={m}", got, xh.astype(np.float64) @ wd, max_outside=8)
-        t_mm = graph_ms(dev, lambda: [QTensorOps.q_matmul(x, wq, out_dtype=ba.F32) for wq in ws], 16, steps, warmup)
-        mid[f"M={m}"] = {"ms": t_mm, "TFLOP/s": 2.0 * m * k * n / t_mm / 1e9, "frac_mfma": 2.0 * m * k * n / t_mm / 1e9 / BF16_PEAK_TFLOPS,
-                         "weight_GB/s": wb / t_mm / 1e6, "max_normalised_error": rel}
-    out["q4s_mid_batch"] = {"workload": "x[M,4096] bf16 x Q4S block-32 PackedU32 [4096,14336] -> f32, 64 to 512 rows (C5's operand types)",
-                            "parity": "vs float64 on every 37th column, rel 1e-2; at most 8 outputs outside burn's elementwise rule "
-                                      "(the tiled kernel rounds s * q to bf16)", **mid}
-    del ws, w0, blob, values, scales
-    dev.trim()
-
-    # ---- scale dtypes: quantize_dynamic + dequantize of C2's tensor ------------------------------
-    rows = 8192
-    nel = rows * 8192
-    host = normal_f32(0xC2, (rows, 8192), outliers=True)
-    xs = [FloatOps.float_from_data(np.roll(host, i * 977, axis=0), dev) for i in range(5)]
-    small = np.ascontiguousarray(host[:256])
-    codes = {ScaleDtype.F16: co.SCALE_F16, ScaleDtype.BF16: co.SCALE_BF16, ScaleDtype.UE4M3: co.SCALE_UE4M3}
-    osch = co.Scheme.make(co.Q8S, [32], co.STORE_PACKED_U32)
-    sd = {}
-    for name, sdt, two in (("f16", ScaleDtype.F16, False), ("bf16", ScaleDtype.BF16, False), ("ue4m3", ScaleDtype.UE4M3, False),
-                           ("f16 under f32", ScaleDtype.F16, True), ("ue4m3 under f32", ScaleDtype.UE4M3, True)):
-        scheme = QuantScheme().per_block((32,), sdt)
-        if two:
-            scheme = scheme.per_tensor(ScaleDtype.F32)
-        tq = QTensorOps.quantize_dynamic(FloatOps.float_from_data(small, dev), scheme)
-        if two:
-            q_ref, stored, g, eff = co.quantize_dynamic_two_level(small, osch, codes[sdt])
-            want = co.encode_two_level(q_ref, osch, stored, g, codes[sdt])
-        else:
-            lo, hi = co.compute_range(small, osch)
-            eff = co.scale_to_dtype(co.compute_q_params(lo, hi, osch.value), codes[sdt])
-            q_ref = co.quantize(small, osch, eff)
-            want = co.encode_with_scale_dtype(q_ref, osch, eff, codes[sdt])
-        if QTensorOps.q_into_data(tq).bytes.tobytes() != want.tobytes():
-            raise ParityError(f"{name} scales: the blob differs from the CPU oracle's")
-        if FloatOps.float_into_data(QTensorOps.dequantize(tq)).tobytes() != co.dequantize(q_ref, osch, eff).tobytes():
-            raise ParityError(f"{name} scales: dequantize differs from the CPU oracle")
-        t_q = graph_ms(dev, lambda: [QTensorOps.quantize_dynamic(xs[i % 5], scheme) for i in range(10)], 10, steps, warmup)
-        qs = [QTensorOps.quantize_dynamic(xs[i % 5], scheme) for i in range(16)]
-        t_d = graph_ms(dev, lambda: [QTensorOps.dequantize(q) for q in qs], 16, steps, warmup)
-        del qs
-        b = 4 * nel + nel + sdt.size() * nel // 32 + (4 if two else 0)
-        sd[name] = {"quantize_dynamic": {"ms": t_q, "GB/s": b / t_q / 1e6, "frac_hbm": b / t_q / 1e6 / HBM_PEAK_GBS},
-                    "dequantize": {"ms": t_d, "GB/s": b / t_d / 1e6, "frac_hbm": b / t_d / 1e6 / HBM_PEAK_GBS}, "bytes": b}
+    if NEXT_PART in ("all", "matmul"):
+        # ---- quantized Linear: the bias rides in the product's epilogue ------------------------------
+        k, n = 4096, 14336
+        w0 = quantized_weight(ba, dev, 0xC4, (k, n), QuantValue.Q8S)
+        blob = QTensorOps.q_into_data(w0)
+        ws = [w0] + [QTensorOps.q_from_data(blob, dev) for _ in range(15)]
+        values, scales = blob.split()
+        bias_h = rng.standard_normal(n, dtype=np.float32)
+        bias = FloatOps.float_from_data(bias_h, dev)
+        cols = np.arange(0, n, 37)
+        wd = unpack_columns(values, scales, k, n, cols, q4=False)
+        lin = {}
+        for m in (1, 16):
+            xh = rng.standard_normal((m, k), dtype=np.float32)
+            x = FloatOps.float_from_data(xh, dev)
+            got = FloatOps.float_into_data(ModuleOps.linear(x, ws[3], bias))[:, cols]
+            matmul_gate(f"linear M={m}", got, xh.astype(np.float64) @ wd + bias_h[cols].astype(np.float64))
+            t_lin = graph_ms(dev, lambda: [ModuleOps.linear(x, wq, bias) for wq in ws], 16, steps, warmup)
+            t_mm = graph_ms(dev, lambda: [QTensorOps.q_matmul(x, wq) for wq in ws], 16, steps, warmup)
+            lin[f"M={m}"] = {"ms": t_lin, "ms_without_bias": t_mm, "GB/s": (k * n + 4 * k * n // 32) / t_lin / 1e6}
+        out["linear"] = {"workload": "x[M,4096] f32 x Q8S block-32 [4096,14336] + bias[14336] -> f32 (C4's weight)",
+                         "parity": "vs float64 on every 37th column, rel 1e-2 and burn's elementwise rule", **lin}
+        # ---- QuantPropagation::Propagate: the product comes back quantized with the weight's scheme -----
+        osch = co.Scheme.make(co.Q8S, [32], co.STORE_PACKED_U32)
+        scheme = ws[0].scheme
+        prop = {}
+        for m in (4, 16):
+            x = FloatOps.float_from_data(rng.standard_normal((m, k), dtype=np.float32), dev)
+            prod = FloatOps.float_into_data(QTensorOps.q_matmul(x, ws[2]))
+            q_ref, s_ref = co.quantize_dynamic(prod, osch)
+            if QTensorOps.q_into_data(QTensorOps.q_matmul_propagate(x, ws[2])).bytes.tobytes() != co.encode(q_ref, osch, s_ref).tobytes():
+                raise ParityError(f"Propagate M={m}: differs from the CPU oracle's quantization of the product")
+            t_p = graph_ms(dev, lambda: [QTensorOps.q_matmul_propagate(x, wq) for wq in ws], 16, steps, warmup)
+            t_2 = graph_ms(dev, lambda: [QTensorOps.quantize_dynamic(QTensorOps.q_matmul(x, wq), scheme) for wq in ws], 16, steps, warmup)
+            prop[f"M={m}"] = {"ms": t_p, "ms_product_then_quantize_dynamic": t_2}
+        out["propagate"] = {"workload": "x[M,4096] f32 x Q8S block-32 [4096,14336] -> Q8S block-32 [M,14336] (C4's weight; the K-slice "
+                                        "reduction quantizes what it sums)",
+                            "parity": "blob bit-exact vs the CPU oracle's quantize_dynamic of the device's float product", **prop}
+        del ws, w0, blob, values, scales
         dev.trim()
-    out["scale_dtypes"] = {"workload": "C2's tensor, Q8S block-32 PackedU32, block scales stored as f16 / bf16 / ue4m3, alone or "
-                                       "relative to an f32 per-tensor scale (two launches more: the largest scale, the split)",
-                           "parity": "blob and dequantized floats bit-exact vs CPU oracle on a 256-row tensor of the same data", **sd}
 
-    # ---- the full-range value of the reference's default scheme --------------------------------------
-    osch_f = co.Scheme.make(co.Q8F, [32], co.STORE_PACKED_U32)
-    scheme_f = QuantScheme(value=QuantValue.Q8F).per_block((32,))
-    tq = QTensorOps.quantize_dynamic(FloatOps.float_from_data(small, dev), scheme_f)
-    q_ref, s_ref = co.quantize_dynamic(small, osch_f)
-    if QTensorOps.q_into_data(tq).bytes.tobytes() != co.encode(q_ref, osch_f, s_ref).tobytes() or \
-            FloatOps.float_into_data(QTensorOps.dequantize(tq)).tobytes() != co.dequantize(q_ref, osch_f, s_ref).tobytes():
-        raise ParityError("Q8F: blob or dequantized floats differ from the CPU oracle's")
-    t_q = graph_ms(dev, lambda: [QTensorOps.quantize_dynamic(xs[i % 5], scheme_f) for i in range(10)], 10, steps, warmup)
-    b = 4 * nel + nel + 4 * nel // 32
-    out["full_range"] = {"workload": "C2's tensor, Q8F (-128..127, span 255) block-32 PackedU32, f32 scales: quantize_dynamic",
-                         "parity": "blob and dequantized floats bit-exact vs CPU oracle on a 256-row tensor of the same data",
-                         "quantize_dynamic": {"ms": t_q, "GB/s": b / t_q / 1e6, "frac_hbm": b / t_q / 1e6 / HBM_PEAK_GBS}, "bytes": b}
-    dev.trim()
+        # ---- the same products over a 4-bit weight ------------------------------------------------------
+        w0 = quantized_weight(ba, dev, 0xC4, (k, n), QuantValue.Q4S)
+        blob = QTensorOps.q_into_data(w0)
+        ws = [w0] + [QTensorOps.q_from_data(blob, dev) for _ in range(15)]
+        values, scales = blob.split()
+        wd = unpack_columns(values, scales, k, n, cols, q4=True)
+        q4 = {}
+        for m in (1, 4, 16):
+            xh = rng.standard_normal((m, k), dtype=np.float32)
+            x = FloatOps.float_from_data(xh, dev)
+            got = FloatOps.float_into_data(QTensorOps.q_matmul(x, ws[5]))[:, cols]
+            rel = matmul_gate(f"Q4S M={m}", got, xh.astype(np.float64) @ wd)
+            t_mm = graph_ms(dev, lambda: [QTensorOps.q_matmul(x, wq) for wq in ws], 16, steps, warmup)
+            wb = k * n // 2 + 4 * k * n // 32
+            q4[f"M={m}"] = {"ms": t_mm, "weight_GB/s": wb / t_mm / 1e6, "frac_hbm": wb / t_mm / 1e6 / HBM_PEAK_GBS,
+                            "max_normalised_error": rel}
+        out["q4s_small_batch"] = {"workload": "x[M,4096] f32 x Q4S block-32 PackedU32 [4096,14336] -> f32 (C4's shape, half the weight bytes)",
+                                  "parity": "vs float64 on every 37th column, rel 1e-2 and burn's elementwise rule", **q4}
+        # batches between the decode kernels (M <= 32) and prefill: the tiled kernel on row tiles it does not fill
+        mid = {}
+        for m in (64, 128, 512):
+            xh = ba.f32_from_bf16_bits(ba.bf16_bits_from_f32(rng.standard_normal((m, k), dtype=np.float32))).reshape(m, k)
+            x = FloatOps.float_from_data(ba.bf16_bits_from_f32(xh), dev, ba.BF16)
+            got = FloatOps.float_into_data(QTensorOps.q_matmul(x, ws[5], out_dtype=ba.F32))[:, cols]
+            rel = matmul_gate(f"Q4S M={m}", got, xh.astype(np.float64) @ wd, max_outside=8)
+            t_mm = graph_ms(dev, lambda: [QTensorOps.q_matmul(x, wq, out_dtype=ba.F32) for wq in ws], 16, steps, warmup)
+            mid[f"M={m}"] = {"ms": t_mm, "TFLOP/s": 2.0 * m * k * n / t_mm / 1e9, "frac_mfma": 2.0 * m * k * n / t_mm / 1e9 / BF16_PEAK_TFLOPS,
+                             "weight_GB/s": wb / t_mm / 1e6, "max_normalised_error": rel}
+        out["q4s_mid_batch"] = {"workload": "x[M,4096] bf16 x Q4S block-32 PackedU32 [4096,14336] -> f32, 64 to 512 rows (C5's operand types)",
+                                "parity": "vs float64 on every 37th column, rel 1e-2; at most 8 outputs outside burn's elementwise rule "
+                                          "(the tiled kernel rounds s * q to bf16)", **mid}
+        del ws, w0, blob, values, scales
+        dev.trim()
 
-    # ---- layout ops on a packed tensor -------------------------------------------------------------
-    scheme = QuantScheme().per_block((32,))
-    tq_small = QTensorOps.quantize_dynamic(FloatOps.float_from_data(small, dev), scheme)
-    q_ref, s_ref = co.quantize_dynamic(small, osch)
-    tr = QTensorOps.q_into_data(QTensorOps.q_swap_dims(tq_small, 0, 1))
-    tv, ts = tr.split()
-    if no.unpack_u32(tv.view(np.uint32), tr.shape, "Q8S").tobytes() != np.ascontiguousarray(q_ref.T).tobytes() or \
-            ts.reshape(-1).tobytes() != np.ascontiguousarray(s_ref.reshape(256, 256).T).tobytes():
-        raise ParityError("swap_dims of a packed block-quantized tensor differs from the oracle's transpose")
-    qs = [QTensorOps.quantize_dynamic(xs[i % 5], scheme) for i in range(8)]
-    t_t = graph_ms(dev, lambda: [QTensorOps.q_swap_dims(q, 0, 1) for q in qs], 8, steps, warmup)
-    b = 2 * (nel + 4 * nel // 32)
-    out["layout"] = {"workload": "q_swap_dims(0, 1) of a Q8S block-32 PackedU32 [8192,8192] tensor: values repacked along "
-                                 "the new last dim, scales moved with their blocks",
-                     "parity": "values and scales bit-exact vs the transposed oracle tensor, 256 x 8192",
-                     "swap_dims": {"ms": t_t, "GB/s": b / t_t / 1e6, "frac_hbm": b / t_t / 1e6 / HBM_PEAK_GBS, "bytes": b}}
-    # ---- integer-domain ops on the same packed tensors ------------------------------------------------
-    from burn_amd import IntOps
-    import burn_amd as _ba
-    idx_h = np.random.default_rng(0x5E1).integers(0, 256, 192)
-    sl = (slice(32, 224), slice(2048, 6144))
-    got = QTensorOps.q_into_data(QTensorOps.q_slice(tq_small, sl))
-    gv, gs = got.split()
-    if no.unpack_u32(gv.view(np.uint32), got.shape, "Q8S").tobytes() != np.ascontiguousarray(q_ref[sl]).tobytes() or \
-            gs.reshape(-1).tobytes() != np.ascontiguousarray(s_ref.reshape(256, 256)[32:224, 64:192]).tobytes():
-        raise ParityError("q_slice of a packed block-quantized tensor differs from the sliced oracle tensor")
-    got = QTensorOps.q_into_data(QTensorOps.q_select(tq_small, 0, IntOps.int_from_data(idx_h.astype(np.int64), dev)))
-    gv, gs = got.split()
-    if no.unpack_u32(gv.view(np.uint32), got.shape, "Q8S").tobytes() != np.ascontiguousarray(q_ref[idx_h]).tobytes() or \
-            gs.reshape(-1).tobytes() != np.ascontiguousarray(s_ref.reshape(256, 256)[idx_h]).tobytes():
-        raise ParityError("q_select of a packed block-quantized tensor differs from the oracle's rows")
-    t_sl = graph_ms(dev, lambda: [QTensorOps.q_slice(q, (slice(1024, 7168), slice(2048, 6144))) for q in qs], 8, steps, warmup)
-    b_sl = 2 * (6144 * 4096 + 4 * 6144 * 4096 // 32)
-    rows_idx = IntOps.int_from_data(np.random.default_rng(0x5E2).integers(0, rows, rows).astype(np.int64), dev)
-    t_se = graph_ms(dev, lambda: [QTensorOps.q_select(q, 0, rows_idx) for q in qs], 8, steps, warmup)
-    b_se = 2 * (nel + 4 * nel // 32) + 8 * rows
-    pt = QuantScheme()                                                   # Q8S per tensor, packed
-    osch_pt = co.Scheme.make(co.Q8S, None, co.STORE_PACKED_U32)
-    q_pt, _ = co.quantize_dynamic(small, osch_pt)
-    am = IntOps.int_into_data(QTensorOps.q_argmax(QTensorOps.quantize_dynamic(FloatOps.float_from_data(small, dev), pt), 1))
-    if am.reshape(-1).tolist() != q_pt.argmax(axis=1).tolist():
-        raise ParityError("q_argmax differs from the first maximum of the oracle's integers")
-    qpt = [QTensorOps.quantize_dynamic(xs[i % 5], pt) for i in range(8)]
-    t_am = graph_ms(dev, lambda: [QTensorOps.q_argmax(q, 1) for q in qpt], 8, steps, warmup)
-    b_am = nel + 8 * rows
-    out["integer_domain"] = {
-        "workload": "q_slice [1024:7168, 2048:6144], q_select of 8192 random rows (dim 0) of a Q8S block-32 PackedU32 [8192,8192] "
-                    "tensor, values and scales moved together; q_argmax along the last dim of the per-tensor one",
-        "parity": "integers and scales bit-exact vs numpy on the oracle's tensor, 256 x 8192",
-        "q_slice": {"ms": t_sl, "GB/s": b_sl / t_sl / 1e6, "frac_hbm": b_sl / t_sl / 1e6 / HBM_PEAK_GBS, "bytes": b_sl},
-        "q_select": {"ms": t_se, "GB/s": b_se / t_se / 1e6, "frac_hbm": b_se / t_se / 1e6 / HBM_PEAK_GBS, "bytes": b_se},
-        "q_argmax": {"ms": t_am, "GB/s": b_am / t_am / 1e6, "frac_hbm": b_am / t_am / 1e6 / HBM_PEAK_GBS, "bytes": b_am}}
-    del qpt, rows_idx
-    dev.trim()
+    if NEXT_PART in ("all", "tensor"):
+        # ---- scale dtypes: quantize_dynamic + dequantize of C2's tensor ------------------------------
+        rows = 8192
+        nel = rows * 8192
+        host = normal_f32(0xC2, (rows, 8192), outliers=True)
+        xs = [FloatOps.float_from_data(np.roll(host, i * 977, axis=0), dev) for i in range(5)]
+        small = np.ascontiguousarray(host[:256])
+        codes = {ScaleDtype.F16: co.SCALE_F16, ScaleDtype.BF16: co.SCALE_BF16, ScaleDtype.UE4M3: co.SCALE_UE4M3}
+        osch = co.Scheme.make(co.Q8S, [32], co.STORE_PACKED_U32)
+        sd = {}
+        for name, sdt, two in (("f16", ScaleDtype.F16, False), ("bf16", ScaleDtype.BF16, False), ("ue4m3", ScaleDtype.UE4M3, False),
+                               ("f16 under f32", ScaleDtype.F16, True), ("ue4m3 under f32", ScaleDtype.UE4M3, True)):
+            scheme = QuantScheme().per_block((32,), sdt)
+            if two:
+                scheme = scheme.per_tensor(ScaleDtype.F32)
+            tq = QTensorOps.quantize_dynamic(FloatOps.float_from_data(small, dev), scheme)
+            if two:
+                q_ref, stored, g, eff = co.quantize_dynamic_two_level(small, osch, codes[sdt])
+                want = co.encode_two_level(q_ref, osch, stored, g, codes[sdt])
+            else:
+                lo, hi = co.compute_range(small, osch)
+                eff = co.scale_to_dtype(co.compute_q_params(lo, hi, osch.value), codes[sdt])
+                q_ref = co.quantize(small, osch, eff)
+                want = co.encode_with_scale_dtype(q_ref, osch, eff, codes[sdt])
+            if QTensorOps.q_into_data(tq).bytes.tobytes() != want.tobytes():
+                raise ParityError(f"{name} scales: the blob differs from the CPU oracle's")
+            if FloatOps.float_into_data(QTensorOps.dequantize(tq)).tobytes() != co.dequantize(q_ref, osch, eff).tobytes():
+                raise ParityError(f"{name} scales: dequantize differs from the CPU oracle")
+            t_q = graph_ms(dev, lambda: [QTensorOps.quantize_dynamic(xs[i % 5], scheme) for i in range(10)], 10, steps, warmup)
+            qs = [QTensorOps.quantize_dynamic(xs[i % 5], scheme) for i in range(16)]
+            t_d = graph_ms(dev, lambda: [QTensorOps.dequantize(q) for q in qs], 16, steps, warmup)
+            del qs
+            b = 4 * nel + nel + sdt.size() * nel // 32 + (4 if two else 0)
+            sd[name] = {"quantize_dynamic": {"ms": t_q, "GB/s": b / t_q / 1e6, "frac_hbm": b / t_q / 1e6 / HBM_PEAK_GBS},
+                        "dequantize": {"ms": t_d, "GB/s": b / t_d / 1e6, "frac_hbm": b / t_d / 1e6 / HBM_PEAK_GBS}, "bytes": b}
+            dev.trim()
+        out["scale_dtypes"] = {"workload": "C2's tensor, Q8S block-32 PackedU32, block scales stored as f16 / bf16 / ue4m3, alone or "
+                                           "relative to an f32 per-tensor scale (two launches more: the largest scale, the split)",
+                               "parity": "blob and dequantized floats bit-exact vs CPU oracle on a 256-row tensor of the same data", **sd}
 
-    # ---- Calibration::AbsMean: the ranges of a ternary weight ------------------------------------------
-    tsch_am = QuantScheme(value=QuantValue.Q2S)
-    osch_t = co.Scheme.make(co.Q2S, None, co.STORE_PACKED_U32)
-    g_ref = co.compute_range_abs_mean(small, osch_t)[1].reshape(-1)[0]
-    tq_am = QTensorOps.quantize_abs_mean(FloatOps.float_from_data(small, dev), tsch_am)
-    av, a_s = QTensorOps.q_into_data(tq_am).split()
-    g_gpu = a_s.reshape(-1)
-    # the mean is a sum the reference leaves to its backend (no order to match): Tolerance::default() between the
-    # two, then everything computed from the device's own scale bit for bit
-    if abs(float(g_gpu[0]) - float(g_ref)) > 1e-5 * abs(float(g_ref)):    # scale = 2 gamma / 2
-        raise ParityError("AbsMean: gamma differs from the oracle's beyond a rounding of the sum")
-    if no.unpack_u32(av.view(np.uint32), small.shape, "Q2S").tobytes() != co.quantize(small, osch_t, g_gpu.copy()).tobytes():
-        raise ParityError("AbsMean: the integers differ from the oracle's quantize with the same scale")
-    t_am2 = graph_ms(dev, lambda: [QTensorOps.quantize_abs_mean(xs[i % 5], tsch_am) for i in range(10)], 10, steps, warmup)
-    b_am2 = 4 * nel + 4 * nel + nel // 4 + 4
-    out["abs_mean"] = {"workload": "C2's tensor -> Q2S per tensor PackedU32 with Calibration::AbsMean: mean |x| (one pass), then quantize",
-                       "parity": "gamma within 1e-5 of the oracle's f64 mean; integers bit-exact vs the oracle's quantize with the device's scale, 256 x 8192",
-                       "quantize_abs_mean": {"ms": t_am2, "GB/s": b_am2 / t_am2 / 1e6, "frac_hbm": b_am2 / t_am2 / 1e6 / HBM_PEAK_GBS,
-                                             "bytes": b_am2, "note": "two passes over x: 4N + 4N + N/4 bytes"}}
-    del qs, xs
-    dev.trim()
+        # ---- the full-range value of the reference's default scheme --------------------------------------
+        osch_f = co.Scheme.make(co.Q8F, [32], co.STORE_PACKED_U32)
+        scheme_f = QuantScheme(value=QuantValue.Q8F).per_block((32,))
+        tq = QTensorOps.quantize_dynamic(FloatOps.float_from_data(small, dev), scheme_f)
+        q_ref, s_ref = co.quantize_dynamic(small, osch_f)
+        if QTensorOps.q_into_data(tq).bytes.tobytes() != co.encode(q_ref, osch_f, s_ref).tobytes() or \
+                FloatOps.float_into_data(QTensorOps.dequantize(tq)).tobytes() != co.dequantize(q_ref, osch_f, s_ref).tobytes():
+            raise ParityError("Q8F: blob or dequantized floats differ from the CPU oracle's")
+        t_q = graph_ms(dev, lambda: [QTensorOps.quantize_dynamic(xs[i % 5], scheme_f) for i in range(10)], 10, steps, warmup)
+        b = 4 * nel + nel + 4 * nel // 32
+        out["full_range"] = {"workload": "C2's tensor, Q8F (-128..127, span 255) block-32 PackedU32, f32 scales: quantize_dynamic",
+                             "parity": "blob and dequantized floats bit-exact vs CPU oracle on a 256-row tensor of the same data",
+                             "quantize_dynamic": {"ms": t_q, "GB/s": b / t_q / 1e6, "frac_hbm": b / t_q / 1e6 / HBM_PEAK_GBS}, "bytes": b}
+        dev.trim()
 
-    # ---- ternary weights ---------------------------------------------------------------------------
-    wt = normal_f32(0xF4, (k, n), 0.02)
-    tsch = QuantScheme(value=QuantValue.Q2S)
-    tws = [QTensorOps.quantize_dynamic(FloatOps.float_from_data(wt, dev), tsch) for _ in range(8)]
-    tblob = QTensorOps.q_into_data(tws[0])
-    tvals, tscale = tblob.split()
-    q_t = no.unpack_u32(tvals.view(np.uint32), (k, n), "Q2S")
-    tern = {}
-    for m in (1, 16):
-        xh = rng.standard_normal((m, k), dtype=np.float32)
-        x = FloatOps.float_from_data(xh, dev)
-        got = FloatOps.float_into_data(QTensorOps.q_matmul(x, tws[1]))
-        ref = (xh.astype(np.float64) @ q_t[:, cols].astype(np.float64)) * np.float64(tscale.reshape(-1)[0])
-        matmul_gate(f"ternary M={m}", got[:, cols], ref)
-        t = graph_ms(dev, lambda: [QTensorOps.q_matmul(x, wq) for wq in tws], 8, steps, warmup)
-        tb = k * n // 4 + 4
-        tern[f"M={m}"] = {"ms": t, "GB/s": tb / t / 1e6, "frac_hbm": tb / t / 1e6 / HBM_PEAK_GBS}
-    out["ternary"] = {"workload": "x[M,4096] f32 x Q2S per-tensor PackedU32 [4096,14336] (16 values per word) -> f32",
-                      "parity": "vs float64 on every 37th column, rel 1e-2 and burn's elementwise rule", **tern}
-    del tws
-    dev.trim()
+        # ---- layout ops on a packed tensor -------------------------------------------------------------
+        scheme = QuantScheme().per_block((32,))
+        tq_small = QTensorOps.quantize_dynamic(FloatOps.float_from_data(small, dev), scheme)
+        q_ref, s_ref = co.quantize_dynamic(small, osch)
+        tr = QTensorOps.q_into_data(QTensorOps.q_swap_dims(tq_small, 0, 1))
+        tv, ts = tr.split()
+        if no.unpack_u32(tv.view(np.uint32), tr.shape, "Q8S").tobytes() != np.ascontiguousarray(q_ref.T).tobytes() or \
+                ts.reshape(-1).tobytes() != np.ascontiguousarray(s_ref.reshape(256, 256).T).tobytes():
+            raise ParityError("swap_dims of a packed block-quantized tensor differs from the oracle's transpose")
+        qs = [QTensorOps.quantize_dynamic(xs[i % 5], scheme) for i in range(8)]
+        t_t = graph_ms(dev, lambda: [QTensorOps.q_swap_dims(q, 0, 1) for q in qs], 8, steps, warmup)
+        b = 2 * (nel + 4 * nel // 32)
+        out["layout"] = {"workload": "q_swap_dims(0, 1) of a Q8S block-32 PackedU32 [8192,8192] tensor: values repacked along "
+                                     "the new last dim, scales moved with their blocks",
+                         "parity": "values and scales bit-exact vs the transposed oracle tensor, 256 x 8192",
+                         "swap_dims": {"ms": t_t, "GB/s": b / t_t / 1e6, "frac_hbm": b / t_t / 1e6 / HBM_PEAK_GBS, "bytes": b}}
+        # ---- integer-domain ops on the same packed tensors ------------------------------------------------
+        from burn_amd import IntOps
+        import burn_amd as _ba
+        idx_h = np.random.default_rng(0x5E1).integers(0, 256, 192)
+        sl = (slice(32, 224), slice(2048, 6144))
+        got = QTensorOps.q_into_data(QTensorOps.q_slice(tq_small, sl))
+        gv, gs = got.split()
+        if no.unpack_u32(gv.view(np.uint32), got.shape, "Q8S").tobytes() != np.ascontiguousarray(q_ref[sl]).tobytes() or \
+                gs.reshape(-1).tobytes() != np.ascontiguousarray(s_ref.reshape(256, 256)[32:224, 64:192]).tobytes():
+            raise ParityError("q_slice of a packed block-quantized tensor differs from the sliced oracle tensor")
+        got = QTensorOps.q_into_data(QTensorOps.q_select(tq_small, 0, IntOps.int_from_data(idx_h.astype(np.int64), dev)))
+        gv, gs = got.split()
+        if no.unpack_u32(gv.view(np.uint32), got.shape, "Q8S").tobytes() != np.ascontiguousarray(q_ref[idx_h]).tobytes() or \
+                gs.reshape(-1).tobytes() != np.ascontiguousarray(s_ref.reshape(256, 256)[idx_h]).tobytes():
+            raise ParityError("q_select of a packed block-quantized tensor differs from the oracle's rows")
+        t_sl = graph_ms(dev, lambda: [QTensorOps.q_slice(q, (slice(1024, 7168), slice(2048, 6144))) for q in qs], 8, steps, warmup)
+        b_sl = 2 * (6144 * 4096 + 4 * 6144 * 4096 // 32)
+        rows_idx = IntOps.int_from_data(np.random.default_rng(0x5E2).integers(0, rows, rows).astype(np.int64), dev)
+        t_se = graph_ms(dev, lambda: [QTensorOps.q_select(q, 0, rows_idx) for q in qs], 8, steps, warmup)
+        b_se = 2 * (nel + 4 * nel // 32) + 8 * rows
+        pt = QuantScheme()                                                   # Q8S per tensor, packed
+        osch_pt = co.Scheme.make(co.Q8S, None, co.STORE_PACKED_U32)
+        q_pt, _ = co.quantize_dynamic(small, osch_pt)
+        am = IntOps.int_into_data(QTensorOps.q_argmax(QTensorOps.quantize_dynamic(FloatOps.float_from_data(small, dev), pt), 1))
+        if am.reshape(-1).tolist() != q_pt.argmax(axis=1).tolist():
+            raise ParityError("q_argmax differs from the first maximum of the oracle's integers")
+        qpt = [QTensorOps.quantize_dynamic(xs[i % 5], pt) for i in range(8)]
+        t_am = graph_ms(dev, lambda: [QTensorOps.q_argmax(q, 1) for q in qpt], 8, steps, warmup)
+        b_am = nel + 8 * rows
+        out["integer_domain"] = {
+            "workload": "q_slice [1024:7168, 2048:6144], q_select of 8192 random rows (dim 0) of a Q8S block-32 PackedU32 [8192,8192] "
+                        "tensor, values and scales moved together; q_argmax along the last dim of the per-tensor one",
+            "parity": "integers and scales bit-exact vs numpy on the oracle's tensor, 256 x 8192",
+            "q_slice": {"ms": t_sl, "GB/s": b_sl / t_sl / 1e6, "frac_hbm": b_sl / t_sl / 1e6 / HBM_PEAK_GBS, "bytes": b_sl},
+            "q_select": {"ms": t_se, "GB/s": b_se / t_se / 1e6, "frac_hbm": b_se / t_se / 1e6 / HBM_PEAK_GBS, "bytes": b_se},
+            "q_argmax": {"ms": t_am, "GB/s": b_am / t_am / 1e6, "frac_hbm": b_am / t_am / 1e6 / HBM_PEAK_GBS, "bytes": b_am}}
+        del qpt, rows_idx
+        dev.trim()
 
-    # ---- a burnpack file to the device -------------------------------------------------------------
-    w3 = quantized_weight(ba, dev, 0xC3, (14336, 4096), QuantValue.Q4S)
-    want = QTensorOps.q_into_data(w3).bytes.tobytes()
-    wr = PackWriter()
-    wr.add_tensor("mlp.up_proj.weight", w3)
-    with tempfile.TemporaryDirectory() as tmp:
-        path = os.path.join(tmp, "c3.bpk")
-        wr.write_to_file(path)
-        size = os.path.getsize(path)
-        best = None
-        for _ in range(3):
-            t0 = time.perf_counter()
-            rd = PackReader(path)
-            t = rd.load("mlp.up_proj.weight", dev)
-            dev.sync()
-            dt = time.perf_counter() - t0
-            rd.close()
-            best = dt if best is None else min(best, dt)
-        if QTensorOps.q_into_data(t).bytes.tobytes() != want:
-            raise ParityError("the tensor loaded from the burnpack file differs from the one written")
-    out["burnpack"] = {"workload": "C3's weight (Q4S block-32 [14336,4096]) written to a burnpack file and loaded back to the "
-                                   "device: open, parse, one host-to-device copy of values || scales",
-                       "parity": "blob of the loaded tensor byte-identical to the written one's",
-                       "file_bytes": size, "load_ms": best * 1e3, "GB/s": size / best / 1e9,
-                       "note": "host path (page cache + PCIe), not an HBM figure"}
+        # ---- Calibration::AbsMean: the ranges of a ternary weight ------------------------------------------
+        tsch_am = QuantScheme(value=QuantValue.Q2S)
+        osch_t = co.Scheme.make(co.Q2S, None, co.STORE_PACKED_U32)
+        g_ref = co.compute_range_abs_mean(small, osch_t)[1].reshape(-1)[0]
+        tq_am = QTensorOps.quantize_abs_mean(FloatOps.float_from_data(small, dev), tsch_am)
+        av, a_s = QTensorOps.q_into_data(tq_am).split()
+        g_gpu = a_s.reshape(-1)
+        # the mean is a sum the reference leaves to its backend (no order to match): Tolerance::default() between the
+        # two, then everything computed from the device's own scale bit for bit
+        if abs(float(g_gpu[0]) - float(g_ref)) > 1e-5 * abs(float(g_ref)):    # scale = 2 gamma / 2
+            raise ParityError("AbsMean: gamma differs from the oracle's beyond a rounding of the sum")
+        if no.unpack_u32(av.view(np.uint32), small.shape, "Q2S").tobytes() != co.quantize(small, osch_t, g_gpu.copy()).tobytes():
+            raise ParityError("AbsMean: the integers differ from the oracle's quantize with the same scale")
+        t_am2 = graph_ms(dev, lambda: [QTensorOps.quantize_abs_mean(xs[i % 5], tsch_am) for i in range(10)], 10, steps, warmup)
+        b_am2 = 4 * nel + 4 * nel + nel // 4 + 4
+        out["abs_mean"] = {"workload": "C2's tensor -> Q2S per tensor PackedU32 with Calibration::AbsMean: mean |x| (one pass), then quantize",
+                           "parity": "gamma within 1e-5 of the oracle's f64 mean; integers bit-exact vs the oracle's quantize with the device's scale, 256 x 8192",
+                           "quantize_abs_mean": {"ms": t_am2, "GB/s": b_am2 / t_am2 / 1e6, "frac_hbm": b_am2 / t_am2 / 1e6 / HBM_PEAK_GBS,
+                                                 "bytes": b_am2, "note": "two passes over x: 4N + 4N + N/4 bytes"}}
+        del qs, xs
+        dev.trim()
+
+    if NEXT_PART in ("all", "matmul"):  # (continued: ternary weights, burnpack)
+        # ---- ternary weights ---------------------------------------------------------------------------
+        wt = normal_f32(0xF4, (k, n), 0.02)
+        tsch = QuantScheme(value=QuantValue.Q2S)
+        tws = [QTensorOps.quantize_dynamic(FloatOps.float_from_data(wt, dev), tsch) for _ in range(8)]
+        tblob = QTensorOps.q_into_data(tws[0])
+        tvals, tscale = tblob.split()
+        q_t = no.unpack_u32(tvals.view(np.uint32), (k, n), "Q2S")
+        tern = {}
+        for m in (1, 16):
+            xh = rng.standard_normal((m, k), dtype=np.float32)
+            x = FloatOps.float_from_data(xh, dev)
+            got = FloatOps.float_into_data(QTensorOps.q_matmul(x, tws[1]))
+            ref = (xh.astype(np.float64) @ q_t[:, cols].astype(np.float64)) * np.float64(tscale.reshape(-1)[0])
+            matmul_gate(f"ternary M={m}", got[:, cols], ref)
+            t = graph_ms(dev, lambda: [QTensorOps.q_matmul(x, wq) for wq in tws], 8, steps, warmup)
+            tb = k * n // 4 + 4
+            tern[f"M={m}"] = {"ms": t, "GB/s": tb / t / 1e6, "frac_hbm": tb / t / 1e6 / HBM_PEAK_GBS}
+        out["ternary"] = {"workload": "x[M,4096] f32 x Q2S per-tensor PackedU32 [4096,14336] (16 values per word) -> f32",
+                          "parity": "vs float64 on every 37th column, rel 1e-2 and burn's elementwise rule", **tern}
+        del tws
+        dev.trim()
+
+        # ---- a burnpack file to the device -------------------------------------------------------------
+        w3 = quantized_weight(ba, dev, 0xC3, (14336, 4096), QuantValue.Q4S)
+        want = QTensorOps.q_into_data(w3).bytes.tobytes()
+        wr = PackWriter()
+        wr.add_tensor("mlp.up_proj.weight", w3)
+        with tempfile.TemporaryDirectory() as tmp:
+            path = os.path.join(tmp, "c3.bpk")
+            wr.write_to_file(path)
+            size = os.path.getsize(path)
+            best = None
+            for _ in range(3):
+                t0 = time.perf_counter()
+                rd = PackReader(path)
+                t = rd.load("mlp.up_proj.weight", dev)
+                dev.sync()
+                dt = time.perf_counter() - t0
+                rd.close()
+                best = dt if best is None else min(best, dt)
+            if QTensorOps.q_into_data(t).bytes.tobytes() != want:
+                raise ParityError("the tensor loaded from the burnpack file differs from the one written")
+        out["burnpack"] = {"workload": "C3's weight (Q4S block-32 [14336,4096]) written to a burnpack file and loaded back to the "
+                                       "device: open, parse, one host-to-device copy of values || scales",
+                           "parity": "blob of the loaded tensor byte-identical to the written one's",
+                           "file_bytes": size, "load_ms": best * 1e3, "GB/s": size / best / 1e9,
+                           "note": "host path (page cache + PCIe), not an HBM figure"}
     return out
 
 
@@ -886,7 +890,7 @@ def cpu_baseline_c2(passes=5):
 
 
 def main():
-    global C5_N
+    global C5_N, NEXT_PART
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=20)
@@ -894,9 +898,12 @@ def main():
     ap.add_argument("--no-others", action="store_true", help="skip the C1/C3/C4/C5 side measurements")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline legs")
     ap.add_argument("--only", default="", help="comma list of side configs to run (c1,c3,c4,c5,next,reference_bench)")
+    ap.add_argument("--next-part", default="all", choices=["all", "matmul", "tensor"],
+                    help="run only one half of the `next` legs (a profiler may not survive all of their graphs in one process)")
     ap.add_argument("--c5-n", type=int, default=C5_N, help="weight columns of the C5 side measurement (default: C5's 14336)")
     args = ap.parse_args()
     C5_N = args.c5_n
+    NEXT_PART = args.next_part
     if args.gpus != 1:
         print("bench.py: this path runs on ONE GPU (the kernels shard by rows / columns with no "
               "exchange; no multi-GPU figure is produced). Run with --gpus 1.", file=sys.stderr)
